@@ -1,0 +1,151 @@
+/*
+ * megafold_amd — C ABI of the MI355X (gfx950) kernels that replace MegaFold's three fused
+ * training kernels.  Plain pointers and sizes only; every pointer that names tensor data is a
+ * DEVICE pointer, every stride is in ELEMENTS.  Nothing here allocates, frees or synchronises:
+ * outputs and workspaces are caller-owned, work is enqueued on the caller's stream (a hipStream_t
+ * passed as void*; NULL = the default stream).
+ *
+ * Return value of every int function: 0 = enqueued; < 0 = argument rejected before anything was
+ * launched (MF_ERR_*, text in mf_last_error()); > 0 = the hipError_t a launch returned.
+ *
+ * Reference interfaces replaced (paths relative to the MegaFold repository):
+ *   mf_evoattn_fwd        EvoformerAttention.forward   megafold/model/FusedEvoAttention/evoattention.py:688-779
+ *   mf_evoattn_bwd        EvoformerAttention.backward  megafold/model/FusedEvoAttention/evoattention.py:782-903
+ *   mf_lnlinear_fwd       layernorm_linear_forward     megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:351-405
+ *   mf_lnlinear_bwd       layernorm_linear_backward    megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:408-474
+ *   mf_swiglu_fwd / _bwd  swiglu_forward / _backward   megafold/model/FusedTransition/fused_transition.py:55-93
+ *   mf_ln_swiglu_fwd/_bwd LayernormLinear + FusedSwiGLU of FusedTransition.ff[0:2]
+ *                                                      megafold/model/FusedTransition/fused_transition.py:128-131
+ */
+#ifndef MEGAFOLD_AMD_H
+#define MEGAFOLD_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+#define MF_DTYPE_F32 0
+#define MF_DTYPE_F16 1
+#define MF_DTYPE_BF16 2
+#define MF_DTYPE_BOOL 3 /* 1 byte per element; only for the attention key mask (true = keep) */
+
+/* argument errors */
+#define MF_ERR_NULL (-1)      /* required pointer is NULL */
+#define MF_ERR_SHAPE (-2)     /* non-positive or unsupported dimension */
+#define MF_ERR_DTYPE (-3)     /* unknown / unsupported element type */
+#define MF_ERR_STRIDE (-4)    /* stride not supported (alignment) */
+#define MF_ERR_ALIGN (-5)     /* pointer not 16-byte aligned */
+#define MF_ERR_WORKSPACE (-6) /* workspace missing or too small */
+
+int mf_version(void);
+/* Text of the last argument error on the calling thread ("" if none). */
+const char* mf_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Pair-biased, key-masked attention ("EvoAttention").
+ *   q, k, v, o, dO, dq, dk, dv : [B, N, S, H, D], element type `dtype`, D contiguous;
+ *                                *_stride = element strides of the (B, N, S, H) axes.
+ *   bias  : [B, 1, H, S, S] of bias_dtype, bias_stride = strides of (B, H, S_query, S_key).
+ *   mask  : [B, N, 1, 1, S] of mask_dtype, ADDED to the logits (0 / -1e9 / -inf ...);
+ *           mask_stride = strides of (B, N, S_key); stride 0 broadcasts.  MF_DTYPE_BOOL is a
+ *           keep-mask: true -> 0, false -> -inf.
+ *   lse   : [B, N, H, S] fp32, written by fwd, read by bwd.
+ *   dbias : [B, H, S, S] fp32 contiguous, written by bwd; NULL = the bias needs no gradient.
+ * Supported: D multiple of 8, D <= 64; dtype f32 / f16 / bf16; strides of q..dv multiples of
+ * 16 bytes; pointers 16-byte aligned.
+ * A query row whose keys are all masked with -inf yields o = 0, lse = -inf and zero gradients.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct mf_evoattn_args {
+  int32_t B, N, S, H, D;
+  int32_t dtype, bias_dtype, mask_dtype;
+  float scale; /* softmax scale; the reference uses D^-0.5 */
+  int32_t reserved0;
+  const void *q, *k, *v;
+  const void* bias;
+  const void* mask;
+  void* o;
+  float* lse;
+  int64_t q_stride[4], k_stride[4], v_stride[4], o_stride[4];
+  int64_t bias_stride[4];
+  int64_t mask_stride[3];
+  /* backward only */
+  const void* dO;
+  void *dq, *dk, *dv;
+  float* dbias;
+  int64_t do_stride[4], dq_stride[4], dk_stride[4], dv_stride[4];
+  /* scratch */
+  void* workspace;
+  uint64_t workspace_bytes;
+  void* stream;
+} mf_evoattn_args;
+
+uint64_t mf_evoattn_fwd_workspace_bytes(const mf_evoattn_args* a);
+uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a);
+int mf_evoattn_fwd(const mf_evoattn_args* a);
+int mf_evoattn_bwd(const mf_evoattn_args* a);
+
+/* ------------------------------------------------------------------------------------------------
+ * LayerNorm -> Linear:  out = LayerNorm(x; gamma, beta, eps) @ W (+ b)
+ *   x     : [M, K] contiguous, element type `dtype`
+ *   gamma : [K], beta : [K] or NULL, W : [K, N] contiguous (the reference's `linear_weight`,
+ *           i.e. nn.Linear.weight transposed), b : [N] or NULL; all of element type `dtype`
+ *   out   : [M, N] contiguous; mean, rstd : [M] fp32 (saved for backward)
+ * Backward: dout [M, N] -> dx [M, K] (dtype); dW [K, N], db [N] (may be NULL), dgamma [K],
+ * dbeta [K] (may be NULL) are fp32.
+ * With act == MF_ACT_SWIGLU (N even): out and dout are [M, N/2] and
+ *   out = silu(u[:, N/2:]) * u[:, :N/2]   with u = LayerNorm(x) @ W   (b must be NULL);
+ * the backward recomputes u, nothing of shape [M, N] is saved.
+ * ---------------------------------------------------------------------------------------------- */
+#define MF_ACT_NONE 0
+#define MF_ACT_SWIGLU 1
+
+typedef struct mf_lnlinear_args {
+  int64_t M;
+  int32_t K, N;
+  int32_t dtype;
+  int32_t act;
+  float eps;
+  int32_t reserved0;
+  const void* x;
+  const void* gamma;
+  const void* beta;
+  const void* W;
+  const void* b;
+  void* out;
+  float* mean;
+  float* rstd;
+  /* backward only */
+  const void* dout;
+  void* dx;
+  float* dW;
+  float* db;
+  float* dgamma;
+  float* dbeta;
+  /* scratch */
+  void* workspace;
+  uint64_t workspace_bytes;
+  void* stream;
+} mf_lnlinear_args;
+
+uint64_t mf_lnlinear_fwd_workspace_bytes(const mf_lnlinear_args* a);
+uint64_t mf_lnlinear_bwd_workspace_bytes(const mf_lnlinear_args* a);
+int mf_lnlinear_fwd(const mf_lnlinear_args* a);
+int mf_lnlinear_bwd(const mf_lnlinear_args* a);
+
+/* ------------------------------------------------------------------------------------------------
+ * SwiGLU on its own (FusedTransition with include_ln=False or use_layernormlinear=False):
+ *   x [M, 2*Dh] contiguous -> y [M, Dh],  y = silu(x[:, Dh:]) * x[:, :Dh]
+ *   backward: dy [M, Dh], x -> dx [M, 2*Dh] = [dy * silu(g), dy * a * (sig(g) + silu(g)(1 - sig(g)))]
+ * dx may alias x (the reference overwrites its saved input, fused_transition.py:49-52).
+ * ---------------------------------------------------------------------------------------------- */
+int mf_swiglu_fwd(const void* x, void* y, int64_t M, int32_t Dh, int32_t dtype, void* stream);
+int mf_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t M, int32_t Dh, int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEGAFOLD_AMD_H */

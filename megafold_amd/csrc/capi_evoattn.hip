@@ -1,0 +1,174 @@
+// C-ABI entry points of the attention path: argument validation (before any launch, so it can be
+// exercised without a GPU), workspace carving and kernel sequencing.
+// Host side of the reference being replaced: EvoformerAttention.forward / .backward
+// (megafold/model/FusedEvoAttention/evoattention.py:688-779, 782-903).
+#include "../../include/megafold_amd.h"
+#include "capi_common.h"
+#include "common.h"
+#include "evoattn.h"
+
+using namespace mf;
+
+namespace {
+
+struct Plan {
+  bool bias_copy;     // bias must be converted / padded into the workspace
+  int bias_ld;        // row length of the fp32 bias the kernels read
+  uint64_t off_bias, off_delta, off_part, total;
+  int n_chunks, rows_per_chunk;
+};
+
+bool bias_direct(const mf_evoattn_args* a) {
+  return a->bias_dtype == MF_DTYPE_F32 && a->bias_stride[3] == 1 && a->bias_stride[2] % 4 == 0 &&
+         a->bias_stride[1] % 4 == 0 && a->bias_stride[0] % 4 == 0 && a->S % 16 == 0 && aligned16(a->bias);
+}
+
+Plan make_plan(const mf_evoattn_args* a, bool backward) {
+  Plan pl{};
+  pl.bias_copy = !bias_direct(a);
+  pl.bias_ld = pl.bias_copy ? round_up(a->S, 16) : (int)a->bias_stride[2];
+  uint64_t off = 0;
+  pl.off_bias = off;
+  if (pl.bias_copy) off += align256((uint64_t)a->B * a->H * a->S * pl.bias_ld * 4);
+  pl.n_chunks = 1;
+  pl.rows_per_chunk = a->N;
+  if (backward) {
+    pl.off_delta = off;
+    off += align256((uint64_t)a->B * a->N * a->H * a->S * 4);
+    pl.off_part = off;
+    if (a->dbias) {
+      pl.n_chunks = evo_dbias_chunks(a->B, a->N, a->S, a->H, a->D, a->dtype);
+      pl.rows_per_chunk = (a->N + pl.n_chunks - 1) / pl.n_chunks;
+      if (pl.n_chunks > 1) off += align256((uint64_t)pl.n_chunks * a->B * a->H * a->S * a->S * 4);
+    }
+  }
+  pl.total = off;
+  return pl;
+}
+
+int check_tensor(const char* name, const void* p, const int64_t* st, int esize) {
+  if (!p) return fail(MF_ERR_NULL, "%s is NULL", name);
+  if (!aligned16(p)) return fail(MF_ERR_ALIGN, "%s is not 16-byte aligned", name);
+  const int unit = 16 / esize;
+  for (int i = 0; i < 4; ++i)
+    if (st[i] % unit != 0 || st[i] < 0)
+      return fail(MF_ERR_STRIDE, "%s stride[%d]=%lld is not a non-negative multiple of %d elements", name, i,
+                  (long long)st[i], unit);
+  return 0;
+}
+
+int check_common(const mf_evoattn_args* a) {
+  clear_error();
+  if (!a) return fail(MF_ERR_NULL, "args is NULL");
+  if (a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0)
+    return fail(MF_ERR_SHAPE, "B, N, S, H, D must be positive (got %d %d %d %d %d)", a->B, a->N, a->S, a->H, a->D);
+  if (a->D % 8 != 0 || a->D > 64) return fail(MF_ERR_SHAPE, "D=%d unsupported: need a multiple of 8, at most 64", a->D);
+  if (a->dtype != MF_DTYPE_F32 && a->dtype != MF_DTYPE_F16 && a->dtype != MF_DTYPE_BF16)
+    return fail(MF_ERR_DTYPE, "dtype %d unsupported for q/k/v", a->dtype);
+  if (a->bias_dtype != MF_DTYPE_F32 && a->bias_dtype != MF_DTYPE_F16 && a->bias_dtype != MF_DTYPE_BF16)
+    return fail(MF_ERR_DTYPE, "bias_dtype %d unsupported", a->bias_dtype);
+  if (a->mask_dtype < MF_DTYPE_F32 || a->mask_dtype > MF_DTYPE_BOOL)
+    return fail(MF_ERR_DTYPE, "mask_dtype %d unsupported", a->mask_dtype);
+  const int es = dtype_size(a->dtype);
+  int rc;
+  if ((rc = check_tensor("q", a->q, a->q_stride, es))) return rc;
+  if ((rc = check_tensor("k", a->k, a->k_stride, es))) return rc;
+  if ((rc = check_tensor("v", a->v, a->v_stride, es))) return rc;
+  if ((rc = check_tensor("o", a->o, a->o_stride, es))) return rc;
+  if (!a->bias) return fail(MF_ERR_NULL, "bias is NULL");
+  if (!a->mask) return fail(MF_ERR_NULL, "mask is NULL");
+  if (!a->lse) return fail(MF_ERR_NULL, "lse is NULL");
+  return 0;
+}
+
+EvoTensor tens(const void* p, const int64_t* st) {
+  return EvoTensor{const_cast<void*>(p), st[0], st[1], st[2], st[3]};
+}
+
+int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStream_t stream) {
+  p = EvoParams{};
+  p.B = a->B; p.N = a->N; p.S = a->S; p.H = a->H; p.D = a->D;
+  p.dtype = a->dtype;
+  p.scale = a->scale;
+  p.q = tens(a->q, a->q_stride); p.k = tens(a->k, a->k_stride); p.v = tens(a->v, a->v_stride);
+  p.o = tens(a->o, a->o_stride);
+  p.mask = a->mask; p.mask_dtype = a->mask_dtype;
+  p.mask_sb = a->mask_stride[0]; p.mask_sn = a->mask_stride[1]; p.mask_sj = a->mask_stride[2];
+  p.lse = a->lse;
+  unsigned char* ws = static_cast<unsigned char*>(a->workspace);
+  if (pl.bias_copy) {
+    float* b32 = reinterpret_cast<float*>(ws + pl.off_bias);
+    hipError_t e = launch_bias_to_f32(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
+                                      a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_ld, stream);
+    if (e != hipSuccess) return (int)e;
+    p.bias = b32;
+    p.bias_sb = (int64_t)a->H * a->S * pl.bias_ld;
+    p.bias_sh = (int64_t)a->S * pl.bias_ld;
+    p.bias_ld = pl.bias_ld;
+  } else {
+    p.bias = static_cast<const float*>(a->bias);
+    p.bias_sb = a->bias_stride[0]; p.bias_sh = a->bias_stride[1]; p.bias_ld = a->bias_stride[2];
+  }
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int mf_version(void) { return 100; }
+extern "C" const char* mf_last_error(void) { return last_error_buf(); }
+
+extern "C" uint64_t mf_evoattn_fwd_workspace_bytes(const mf_evoattn_args* a) {
+  if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0) return 0;
+  return make_plan(a, false).total;
+}
+extern "C" uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a) {
+  if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0) return 0;
+  return make_plan(a, true).total;
+}
+
+extern "C" int mf_evoattn_fwd(const mf_evoattn_args* a) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  const Plan pl = make_plan(a, false);
+  if (pl.total > 0 && (!a->workspace || a->workspace_bytes < pl.total))
+    return fail(MF_ERR_WORKSPACE, "forward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
+                (unsigned long long)(a->workspace ? a->workspace_bytes : 0));
+  if (pl.total > 0 && !aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  EvoParams p;
+  rc = fill_params(a, pl, p, stream);
+  if (rc) return rc;
+  return (int)launch_evo_fwd(p, stream);
+}
+
+extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
+  int rc = check_common(a);
+  if (rc) return rc;
+  const int es = dtype_size(a->dtype);
+  if ((rc = check_tensor("dO", a->dO, a->do_stride, es))) return rc;
+  if ((rc = check_tensor("dq", a->dq, a->dq_stride, es))) return rc;
+  if ((rc = check_tensor("dk", a->dk, a->dk_stride, es))) return rc;
+  if ((rc = check_tensor("dv", a->dv, a->dv_stride, es))) return rc;
+  if (a->dbias && !aligned16(a->dbias)) return fail(MF_ERR_ALIGN, "dbias is not 16-byte aligned");
+  const Plan pl = make_plan(a, true);
+  if (!a->workspace || a->workspace_bytes < pl.total)
+    return fail(MF_ERR_WORKSPACE, "backward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
+                (unsigned long long)(a->workspace ? a->workspace_bytes : 0));
+  if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  EvoParams p;
+  rc = fill_params(a, pl, p, stream);
+  if (rc) return rc;
+  unsigned char* ws = static_cast<unsigned char*>(a->workspace);
+  p.dO = tens(a->dO, a->do_stride);
+  p.dq = tens(a->dq, a->dq_stride); p.dk = tens(a->dk, a->dk_stride); p.dv = tens(a->dv, a->dv_stride);
+  p.delta = reinterpret_cast<float*>(ws + pl.off_delta);
+  p.dbias = a->dbias;
+  p.n_chunks = pl.n_chunks;
+  p.rows_per_chunk = pl.rows_per_chunk;
+  p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
+  hipError_t e = launch_evo_bwd_dqkv(p, stream);
+  if (e != hipSuccess) return (int)e;
+  if (a->dbias) e = launch_evo_bwd_dbias(p, stream);
+  return (int)e;
+}

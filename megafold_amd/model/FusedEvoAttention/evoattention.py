@@ -1,0 +1,170 @@
+"""Pair-biased, key-masked attention ("EvoAttention") on MI355X.
+
+Drop-in for the reference module ``megafold/model/FusedEvoAttention/evoattention.py``:
+``TritonEvoformer(Q, K, V, res_mask, pair_bias) -> O`` (evoattention.py:905) and the
+``EvoformerAttention`` autograd function behind it (evoattention.py:688-903).  The name
+``TritonEvoformer`` is kept so call sites (``megafold/model/attention.py:489``) need no change; there
+is no Triton here, the work is done by HIP kernels reached through ``mf_evoattn_fwd`` /
+``mf_evoattn_bwd``.
+
+Shapes (evoattention.py:691-693)::
+
+    Q, K, V    [B, N, S, H, D]      O [B, N, S, H, D] in Q's dtype
+    res_mask   [B, N, 1, 1, S]      added to the logits (0 / -1e9 / -inf); bool = keep-mask
+    pair_bias  [B, 1, H, S, S]
+
+Differences from the reference, all on purpose:
+
+* Q, K, V, dO are consumed in place through their strides and O, dQ, dK, dV are written in the API
+  layout, so the eight ``transpose(-2, -3).contiguous()`` copies (evoattention.py:700-702, 777, 787,
+  899-901) do not exist and nothing transposed is kept for backward.
+* Size-1 batch / row dimensions of ``res_mask`` and ``pair_bias`` broadcast.
+* A ``bool`` mask is a keep-mask (True = attend).  The reference would add 0/1 to the logits
+  (evoattention.py:66), which masks nothing.
+* A query row whose keys are all ``-inf`` gives O = 0 and zero gradients instead of NaN.
+* The bias gradient is reduced in a fixed order without atomics (bitwise reproducible).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from ... import _lib
+
+__all__ = ["EvoformerAttention", "TritonEvoformer", "evoattention_forward", "evoattention_backward"]
+
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def _strided_ok(t: torch.Tensor) -> bool:
+    """Kernel requirement: unit stride on D, other strides multiples of 16 bytes, base aligned."""
+    unit = 16 // t.element_size()
+    return (t.stride(-1) == 1 and all(s % unit == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0)
+
+
+def _prep_qkv(t: torch.Tensor) -> torch.Tensor:
+    return t if _strided_ok(t) else t.contiguous()
+
+
+def _prep_mask(res_mask: torch.Tensor, B: int, N: int, S: int) -> torch.Tensor:
+    if res_mask.dim() != 5 or res_mask.shape[2] != 1 or res_mask.shape[3] != 1 or res_mask.shape[4] != S:
+        raise ValueError("res_mask must be [B, N, 1, 1, S], got %s" % (tuple(res_mask.shape),))
+    if res_mask.dtype not in _FLOATS and res_mask.dtype != torch.bool:
+        res_mask = res_mask.to(torch.float32)
+    return res_mask.expand(B, N, 1, 1, S)
+
+
+def _prep_bias(pair_bias: torch.Tensor, B: int, H: int, S: int) -> torch.Tensor:
+    if pair_bias.dim() != 5 or pair_bias.shape[1] != 1 or tuple(pair_bias.shape[2:]) != (H, S, S):
+        raise ValueError("pair_bias must be [B, 1, H, S, S], got %s" % (tuple(pair_bias.shape),))
+    if pair_bias.dtype not in _FLOATS:
+        pair_bias = pair_bias.to(torch.float32)
+    return pair_bias.expand(B, 1, H, S, S)
+
+
+def _fill_common(a: _lib.EvoAttnArgs, Q, K, V, mask, bias, O, lse) -> None:
+    B, N, S, H, D = Q.shape
+    a.B, a.N, a.S, a.H, a.D = B, N, S, H, D
+    a.dtype = _lib.dtype_code(Q.dtype)
+    a.bias_dtype = _lib.dtype_code(bias.dtype)
+    a.mask_dtype = _lib.dtype_code(mask.dtype)
+    a.scale = float(D) ** -0.5  # evoattention.py:705
+    a.q, a.k, a.v, a.o = Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr()
+    a.bias, a.mask, a.lse = bias.data_ptr(), mask.data_ptr(), lse.data_ptr()
+    a.q_stride = _lib.I64x4(*Q.stride()[:4])
+    a.k_stride = _lib.I64x4(*K.stride()[:4])
+    a.v_stride = _lib.I64x4(*V.stride()[:4])
+    a.o_stride = _lib.I64x4(*O.stride()[:4])
+    bs = bias.stride()
+    a.bias_stride = _lib.I64x4(bs[0], bs[2], bs[3], bs[4])
+    ms = mask.stride()
+    a.mask_stride = _lib.I64x3(ms[0], ms[1], ms[4])
+    a.stream = torch.cuda.current_stream(Q.device).cuda_stream
+
+
+def _check_inputs(Q, K, V) -> None:
+    if Q.dim() != 5:
+        raise ValueError("Q must be [B, N, S, H, D], got %s" % (tuple(Q.shape),))
+    # the reference asserts equal head dims (evoattention.py:695-696)
+    assert Q.shape[-1] == K.shape[-1] and K.shape[-1] == V.shape[-1]
+    if K.shape != Q.shape or V.shape != Q.shape:
+        raise ValueError("Q, K, V must have the same shape")
+    if Q.dtype not in _FLOATS or K.dtype != Q.dtype or V.dtype != Q.dtype:
+        raise TypeError("Q, K, V must share one of float32 / float16 / bfloat16")
+    if not Q.is_cuda:
+        raise RuntimeError("EvoformerAttention runs on the GPU only (got device %s)" % Q.device)
+
+
+def evoattention_forward(Q, K, V, res_mask, pair_bias):
+    """O, LSE = forward.  Returns also the tensors exactly as the kernels saw them."""
+    _check_inputs(Q, K, V)
+    B, N, S, H, D = Q.shape
+    Q, K, V = _prep_qkv(Q), _prep_qkv(K), _prep_qkv(V)
+    mask = _prep_mask(res_mask, B, N, S)
+    bias = _prep_bias(pair_bias, B, H, S)
+    lib = _lib.lib()
+    with torch.cuda.device(Q.device):
+        O = torch.empty((B, N, S, H, D), dtype=Q.dtype, device=Q.device)
+        lse = torch.empty((B, N, H, S), dtype=torch.float32, device=Q.device)
+        a = _lib.EvoAttnArgs()
+        _fill_common(a, Q, K, V, mask, bias, O, lse)
+        nbytes = lib.mf_evoattn_fwd_workspace_bytes(C.byref(a))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device) if nbytes else None
+        a.workspace = ws.data_ptr() if ws is not None else None
+        a.workspace_bytes = nbytes
+        _lib.check(lib.mf_evoattn_fwd(C.byref(a)), "mf_evoattn_fwd")
+    return O, lse, (Q, K, V, mask, bias)
+
+
+def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True):
+    """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state."""
+    B, N, S, H, D = Q.shape
+    if dO.dtype != Q.dtype:
+        dO = dO.to(Q.dtype)
+    dO = _prep_qkv(dO)
+    lib = _lib.lib()
+    with torch.cuda.device(Q.device):
+        dQ = torch.empty((B, N, S, H, D), dtype=Q.dtype, device=Q.device)
+        dK = torch.empty_like(dQ)
+        dV = torch.empty_like(dQ)
+        dbias = torch.empty((B, 1, H, S, S), dtype=torch.float32, device=Q.device) if need_dbias else None
+        a = _lib.EvoAttnArgs()
+        _fill_common(a, Q, K, V, mask, bias, O, lse)
+        a.dO, a.dq, a.dk, a.dv = dO.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr()
+        a.dbias = dbias.data_ptr() if dbias is not None else None
+        a.do_stride = _lib.I64x4(*dO.stride()[:4])
+        a.dq_stride = _lib.I64x4(*dQ.stride()[:4])
+        a.dk_stride = _lib.I64x4(*dK.stride()[:4])
+        a.dv_stride = _lib.I64x4(*dV.stride()[:4])
+        nbytes = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=Q.device)
+        a.workspace = ws.data_ptr()
+        a.workspace_bytes = nbytes
+        _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd")
+    return dQ, dK, dV, dbias
+
+
+class EvoformerAttention(torch.autograd.Function):
+    """Same contract as the reference class of this name (evoattention.py:688-903)."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, res_mask, pair_bias):
+        O, lse, (Qs, Ks, Vs, mask, bias) = evoattention_forward(Q, K, V, res_mask, pair_bias)
+        ctx.save_for_backward(Qs, Ks, Vs, mask, bias, O, lse)
+        ctx.bias_shape = tuple(pair_bias.shape)
+        return O
+
+    @staticmethod
+    def backward(ctx, dO):
+        Q, K, V, mask, bias, O, lse = ctx.saved_tensors
+        need_dbias = ctx.needs_input_grad[4]
+        dQ, dK, dV, dbias = evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias)
+        if dbias is not None:
+            if ctx.bias_shape[0] == 1 and dbias.shape[0] != 1:
+                dbias = dbias.sum(0, keepdim=True)
+            dbias = dbias.to(dO.dtype)  # the reference returns d_pair_bias in dO's dtype (evoattention.py:903)
+        return dQ, dK, dV, None, dbias
+
+
+TritonEvoformer = EvoformerAttention.apply
