@@ -1,0 +1,112 @@
+"""The C-ABI library: loads, exports every symbol the header declares, rejects bad arguments before
+touching the GPU (so this runs without one)."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+from megafold_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "megafold_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(_lib.SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    out = subprocess.run(["nm", "-D", "--defined-only", str(_lib.LIB_PATH)], capture_output=True, text=True).stdout
+    exported = set(re.findall(r"\sT\s+(mf_[a-z0-9_]+)", out))
+    assert set(declared_functions()) <= exported
+    assert lib.mf_version() >= 100
+
+
+def test_header_compiles_as_plain_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "megafold_amd.h"\nint main(void){mf_evoattn_args a; mf_lnlinear_args b; (void)a; (void)b; return 0;}\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src), "-o",
+                    str(tmp_path / "t.o")], check=True)
+
+
+def test_struct_layout_matches_header(tmp_path):
+    src = tmp_path / "s.c"
+    src.write_text('#include <stdio.h>\n#include "megafold_amd.h"\nint main(void){printf("%zu %zu %zu %zu\\n", '
+                   'sizeof(mf_evoattn_args), offsetof(mf_evoattn_args, workspace), sizeof(mf_lnlinear_args), '
+                   'offsetof(mf_lnlinear_args, workspace)); return 0;}\n')
+    exe = tmp_path / "s"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    a, b, c, d = map(int, subprocess.run([str(exe)], capture_output=True, text=True).stdout.split())
+    assert (a, b) == (C.sizeof(_lib.EvoAttnArgs), _lib.EvoAttnArgs.workspace.offset)
+    assert (c, d) == (C.sizeof(_lib.LnLinearArgs), _lib.LnLinearArgs.workspace.offset)
+
+
+def _evo_args():
+    a = _lib.EvoAttnArgs()
+    a.B, a.N, a.S, a.H, a.D = 1, 2, 64, 2, 32
+    a.dtype, a.bias_dtype, a.mask_dtype = _lib.MF_BF16, _lib.MF_F32, _lib.MF_F32
+    a.scale = 32 ** -0.5
+    fake = 0x10000  # never dereferenced: every check below fails before a launch
+    for f in ("q", "k", "v", "o", "bias", "mask", "lse"):
+        setattr(a, f, fake)
+    st = _lib.I64x4(2 * 64 * 2 * 32, 64 * 2 * 32, 2 * 32, 32)
+    a.q_stride = a.k_stride = a.v_stride = a.o_stride = st
+    a.bias_stride = _lib.I64x4(2 * 64 * 64, 64 * 64, 64, 1)
+    a.mask_stride = _lib.I64x3(2 * 64, 64, 1)
+    return a
+
+
+@pytest.mark.parametrize("mutate, code, text", [
+    (lambda a: setattr(a, "q", None), -1, "q is NULL"),
+    (lambda a: setattr(a, "D", 12), -2, "D=12"),
+    (lambda a: setattr(a, "D", 128), -2, "D=128"),
+    (lambda a: setattr(a, "S", 0), -2, "positive"),
+    (lambda a: setattr(a, "dtype", 7), -3, "dtype 7"),
+    (lambda a: setattr(a, "mask_dtype", 9), -3, "mask_dtype"),
+    (lambda a: setattr(a, "k_stride", _lib.I64x4(8192, 4096, 63, 32)), -4, "k stride[2]=63"),
+    (lambda a: setattr(a, "v", 0x10004), -5, "v is not 16-byte aligned"),
+])
+def test_attention_argument_errors(mutate, code, text):
+    lib = _lib.lib()
+    a = _evo_args()
+    mutate(a)
+    assert lib.mf_evoattn_fwd(C.byref(a)) == code
+    assert text in lib.mf_last_error().decode()
+    with pytest.raises(RuntimeError, match="rejected"):
+        _lib.check(code, "mf_evoattn_fwd")
+
+
+def test_attention_workspace_contract():
+    lib = _lib.lib()
+    a = _evo_args()
+    assert lib.mf_evoattn_fwd_workspace_bytes(C.byref(a)) == 0          # fp32 bias is read in place
+    a.bias_dtype = _lib.MF_BF16
+    need = lib.mf_evoattn_fwd_workspace_bytes(C.byref(a))
+    assert need >= 1 * 2 * 64 * 64 * 4
+    assert lib.mf_evoattn_fwd(C.byref(a)) == -6 and "workspace" in lib.mf_last_error().decode()
+    a.bias_dtype = _lib.MF_F32
+    for f in ("dO", "dq", "dk", "dv", "dbias"):
+        setattr(a, f, 0x10000)
+    a.do_stride = a.dq_stride = a.dk_stride = a.dv_stride = a.q_stride
+    bw = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
+    assert bw >= 1 * 2 * 2 * 64 * 4                                      # at least delta
+    assert lib.mf_evoattn_bwd(C.byref(a)) == -6
+
+
+def test_python_wrapper_fails_loudly_without_gpu_tensors():
+    import torch
+    from megafold_amd.model.FusedEvoAttention.evoattention import TritonEvoformer
+    q = torch.zeros(1, 2, 16, 2, 8)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        TritonEvoformer(q, q, q, torch.zeros(1, 2, 1, 1, 16), torch.zeros(1, 1, 2, 16, 16))

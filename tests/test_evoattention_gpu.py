@@ -1,0 +1,195 @@
+"""Parity of the HIP attention path against the CPU oracle (GPU box only).  Every call goes through
+the C ABI (``mf_evoattn_fwd`` / ``mf_evoattn_bwd``) via the Python operator, never through a fallback."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import tol_for
+from megafold_amd import workloads
+from megafold_amd.model.FusedEvoAttention.evoattention import (EvoformerAttention, TritonEvoformer,
+                                                                evoattention_backward, evoattention_forward)
+from oracle import evoattention as oe
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+f64 = torch.float64
+
+
+def to_dev(inp):
+    return {k: v.cuda() for k, v in inp.items()}
+
+
+def run_op(dev, need_bias_grad=True):
+    q, k, v = (dev[n].clone().requires_grad_() for n in "qkv")
+    bias = dev["bias"].clone().requires_grad_(need_bias_grad)
+    out = TritonEvoformer(q, k, v, dev["mask"], bias)
+    out.backward(dev["dO"])
+    return out.detach(), q.grad, k.grad, v.grad, bias.grad
+
+
+def oracle_all(inp, chunk=64):
+    dt = f64 if inp["q"].numel() < 4_000_000 else torch.float32
+    return oe.evo_attention_chunked(inp["q"], inp["k"], inp["v"], inp["mask"], inp["bias"], inp["dO"], chunk=chunk, dtype=dt)
+
+
+def check(got, want, dtype, names=("O", "dQ", "dK", "dV", "dBias")):
+    for name, g, w in zip(names, got, want):
+        assert not torch.isnan(g).any(), name
+        torch.testing.assert_close(g.cpu().to(w.dtype), w, msg=lambda m, n=name: "%s: %s" % (n, m), **tol_for(dtype))
+
+
+# shapes from the reference's sweep (tests/test_evoattention.py:85-135), sized for a quick oracle
+SWEEP = [
+    # B, N, S, H, D, masked, dtype
+    (1, 1, 23, 16, 8, 3, torch.float16),
+    (1, 4, 64, 4, 32, 8, torch.bfloat16),
+    (2, 3, 77, 3, 32, 5, torch.bfloat16),
+    (1, 2, 160, 2, 64, 0, torch.bfloat16),
+    (1, 2, 96, 1, 16, 3, torch.float16),
+    (1, 1, 384, 16, 64, 0, torch.bfloat16),   # single attention with pair bias (N=1, H=16, D=64)
+    (1, 5, 200, 5, 32, 17, torch.bfloat16),
+    (1, 2, 499, 4, 32, 33, torch.bfloat16),
+    (1, 2, 800, 2, 32, 40, torch.bfloat16),   # more key tiles than one chunk of the dQ/dK/dV kernel holds at D=32? no: 25 tiles
+    (1, 1, 1280, 1, 64, 0, torch.bfloat16),   # longest sequence of the reference sweep
+    (1, 3, 50, 2, 8, 3, torch.float32),
+    (1, 2, 130, 2, 64, 9, torch.float32),
+]
+
+
+@pytest.mark.parametrize("B,N,S,H,D,nm,dtype", SWEEP)
+def test_forward_backward_parity(B, N, S, H, D, nm, dtype):
+    print("case", B, N, S, H, D, nm, dtype, flush=True)
+    inp = workloads.evoattention_inputs(B, N, S, H, D, nm, dtype=dtype, seed=S + D)
+    got = run_op(to_dev(inp))
+    check(got, oracle_all(inp), dtype)
+
+
+def test_config1_fp32_forward_against_golden():
+    inp = workloads.config1()
+    dev = to_dev(inp)
+    O, lse, _ = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"])
+    g = np.load(os.path.join(GOLD, "evoattn_c1.npz"))
+    np.testing.assert_allclose(O[0, ::16, ::8].cpu().numpy(), g["o_rows"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(lse[0, ::16, :, ::8].cpu().numpy(), g["lse_rows"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(O.double().sum(dim=(0, 1, 2)).cpu().numpy(), g["o_colsum"], rtol=1e-4, atol=1e-3)
+    # masked keys (last 8) have exactly zero probability: perturbing them changes no bit
+    k2, v2 = dev["k"].clone(), dev["v"].clone()
+    k2[:, :, -8:] += 7.0
+    v2[:, :, -8:] -= 3.0
+    O2, lse2, _ = evoattention_forward(dev["q"], k2, v2, dev["mask"], dev["bias"])
+    assert torch.equal(O, O2) and torch.equal(lse, lse2)
+
+
+def test_small_fp32_backward_against_golden():
+    g = np.load(os.path.join(GOLD, "evoattn_small_bwd.npz"))
+    inp = workloads.evoattention_inputs(2, 3, 45, 2, 16, 7, dtype=torch.float32, seed=3, mask_value=-1e9)
+    got = run_op(to_dev(inp))
+    for name, t in zip(("o", "dq", "dk", "dv", "dbias"), got):
+        np.testing.assert_allclose(t.cpu().numpy(), g[name], rtol=1e-4, atol=1e-5, err_msg=name)
+
+
+def test_config2_full_size_parity_and_properties():
+    """C2: [1, 384, 384, 4, 32] bf16, last 38 keys padded — the headline workload."""
+    inp = workloads.config2()
+    dev = to_dev(inp)
+    got = run_op(dev)
+    check(got, oracle_all(inp, chunk=48), torch.bfloat16)
+    O, dQ, dK, dV, dB = got
+    # masked keys: exactly zero gradient
+    assert torch.count_nonzero(dK[:, :, -38:]) == 0 and torch.count_nonzero(dV[:, :, -38:]) == 0
+    assert torch.count_nonzero(dB[..., -38:]) == 0
+    # rows of dS sum to zero, hence rows of dBias do (sum over 384 rows of bf16-rounded terms)
+    assert dB.float().sum(-1).abs().max() < 0.5
+    # run-to-run bitwise reproducibility (no atomics anywhere)
+    again = run_op(dev)
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
+    # every row n is an independent problem: a slice of rows reproduces the same bits
+    sl = slice(100, 108)
+    O_sl, _, _ = evoattention_forward(dev["q"][:, sl], dev["k"][:, sl], dev["v"][:, sl], dev["mask"][:, sl], dev["bias"])
+    assert torch.equal(O_sl, O[:, sl])
+
+
+@pytest.mark.parametrize("kind", ["-inf", "-1e9", "bool", "bf16", "broadcast", "fully_masked_row"])
+def test_mask_conventions(kind):
+    B, N, S, H, D = 2, 3, 96, 2, 32
+    inp = workloads.evoattention_inputs(B, N, S, H, D, 11, dtype=torch.bfloat16, seed=21)
+    ref_inp = dict(inp)
+    if kind == "-1e9":
+        inp = workloads.evoattention_inputs(B, N, S, H, D, 11, dtype=torch.bfloat16, seed=21, mask_value=-1e9)
+        ref_inp = dict(inp)
+    elif kind == "bool":
+        inp["mask"] = inp["mask"] == 0
+        ref_inp = dict(inp)
+    elif kind == "bf16":
+        inp["mask"] = inp["mask"].to(torch.bfloat16)
+    elif kind == "broadcast":
+        inp["mask"] = inp["mask"][:1, :1].clone()
+        inp["bias"] = inp["bias"][:1].clone()
+        ref_inp = dict(inp, mask=inp["mask"].expand(B, N, 1, 1, S), bias=inp["bias"].expand(B, 1, H, S, S))
+    elif kind == "fully_masked_row":
+        inp["mask"][0, 1] = float("-inf")
+        ref_inp = dict(inp)
+    got = run_op(to_dev(inp))
+    want = list(oe.evo_attention_chunked(ref_inp["q"], ref_inp["k"], ref_inp["v"], ref_inp["mask"], ref_inp["bias"],
+                                         ref_inp["dO"], dtype=f64))
+    if kind == "broadcast":
+        want[4] = want[4].sum(0, keepdim=True)
+    check(got, want, torch.bfloat16)
+    assert torch.count_nonzero(got[2][:, :, -11:]) == 0      # dK at masked keys
+    if kind == "fully_masked_row":
+        assert torch.count_nonzero(got[0][0, 1]) == 0 and torch.count_nonzero(got[1][0, 1]) == 0
+
+
+def test_strided_views_of_a_fused_projection_and_bf16_bias():
+    """q and k/v as the model produces them: views of [B*N, S, H*D] / chunk(2) of [.., 2*H*D]
+    (megafold/model/attention.py:177-182, 469-479), bias in bf16."""
+    B, N, S, H, D = 1, 6, 128, 4, 32
+    inp = workloads.evoattention_inputs(B, N, S, H, D, 9, dtype=torch.bfloat16, seed=5, bias_dtype=torch.bfloat16)
+    dev = to_dev(inp)
+    kv = torch.cat([dev["k"].reshape(B, N, S, H * D), dev["v"].reshape(B, N, S, H * D)], dim=-1)
+    k_view, v_view = (t.reshape(B, N, S, H, D) for t in kv.chunk(2, dim=-1))
+    assert not k_view.is_contiguous()
+    dev2 = dict(dev, k=k_view, v=v_view)
+    got = run_op(dev2)
+    check(got, oracle_all(inp), torch.bfloat16)
+    assert got[4].dtype == torch.bfloat16
+
+
+def test_no_bias_gradient_requested_and_function_signature():
+    inp = workloads.evoattention_inputs(1, 2, 64, 2, 32, 4, dtype=torch.bfloat16, seed=9)
+    dev = to_dev(inp)
+    got = run_op(dev, need_bias_grad=False)
+    assert got[4] is None
+    check(got[:4], oracle_all(inp)[:4], torch.bfloat16)
+    assert TritonEvoformer.__self__ is EvoformerAttention
+    with pytest.raises(AssertionError):   # the reference asserts equal head dims (evoattention.py:695-696)
+        TritonEvoformer(dev["q"], dev["k"][..., :16], dev["v"], dev["mask"], dev["bias"])
+
+
+def test_config5_peak_activation_memory():
+    """C5 [1, 768, 768, 4, 32]: peak extra memory of fwd+bwd stays at the O(N*S*H*D) bound — O, dQ, dK,
+    dV (144 MiB each) + LSE, delta, dBias (9 MiB each) — plus the declared workspace (partial bias
+    gradients, at most 8 x 9 MiB); nothing of size N*H*S*S (6.75 GiB) is ever allocated."""
+    inp = workloads.config5()
+    dev = to_dev(inp)
+    q, k, v = (dev[n].requires_grad_() for n in "qkv")
+    bias = dev["bias"].requires_grad_()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    out = TritonEvoformer(q, k, v, dev["mask"], bias)
+    out.backward(dev["dO"])
+    torch.cuda.synchronize()
+    peak_mib = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+    bound = 4 * 144 + 3 * 9
+    workspace = 8 * 9
+    print("C5 peak activation MiB: %.1f (bound %d + workspace %d)" % (peak_mib, bound, workspace), flush=True)
+    assert peak_mib <= bound + workspace + 1
+    # spot parity on a few rows against the oracle (full-size oracle needs 6.75 GiB of scores)
+    sl = slice(300, 304)
+    Or, _ = oe.evo_attention_forward(inp["q"][:, sl], inp["k"][:, sl], inp["v"][:, sl], inp["mask"][:, sl], inp["bias"])
+    torch.testing.assert_close(out[:, sl].detach().cpu().float(), Or, **tol_for(torch.bfloat16))
+    assert torch.count_nonzero(k.grad[:, :, -96:]) == 0
