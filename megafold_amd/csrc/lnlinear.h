@@ -1,0 +1,59 @@
+// Parameter block and launch entry points of the LayerNorm->Linear (and LayerNorm->SwiGLU) kernels.
+// Replaces the Triton kernels of the reference:
+//   megafold/model/FusedLayernormLinear/fused_layernorm_linear.py
+//     _first_forward_kernel :109-140, _second_forward_kernel :147-218,
+//     _first_backward_kernel :226-308, _second_backward_kernel :311-348
+//   megafold/model/FusedTransition/fused_transition.py  _swiglu_forward_kernel :11-26,
+//     _swiglu_backward_kernel :29-52
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mf {
+
+enum { LN_ACT_NONE = 0, LN_ACT_SWIGLU = 1, LN_ACT_SWIGLU_BWD = 2 };
+
+struct LnParams {
+  int64_t M;
+  int K, N;        // N = columns of W (for SwiGLU the output has N/2 columns)
+  int KP;          // K rounded up to the kernel's padded width
+  int dtype;
+  float eps;
+  const void* x;       // [M, K]
+  const void* gamma;   // [K]
+  const void* beta;    // [K] or null
+  const void* W;       // [K, N]
+  const void* b;       // [N] or null
+  void* out;           // [M, N] (or [M, N/2] with SwiGLU)
+  float* mean;         // [M]
+  float* rstd;         // [M]
+  // prepared weights (workspace)
+  void* Wt;            // [N, KP]  gamma[k] * W[k, n], transposed, element type of x   (forward)
+  void* Wg;            // [K, N]   gamma[k] * W[k, n], element type of x               (backward dx)
+  float* colsum;       // [N] sum_k Wt[n, k]
+  float* bprime;       // [N] sum_k beta[k] W[k, n] + b[n]
+  // backward
+  const void* dout;    // [M, N] (or [M, N/2] with SwiGLU)
+  void* dx;            // [M, K]
+  void* du;            // [M, N] gradient of the pre-activation (SwiGLU backward scratch)
+  float* dW;           // [K, N]
+  float* db;           // [N] or null
+  float* dgamma;       // [K]
+  float* dbeta;        // [K] or null
+  float* Gpart;        // [R, K, N] partial x_hat^T dOut
+  float* spart;        // [R, N]   partial column sums of dOut
+  int R;               // number of row ranges (partials)
+  int64_t rows_per_range;
+};
+
+hipError_t launch_ln_prep(const LnParams& p, bool forward, hipStream_t stream);
+hipError_t launch_ln_fwd(const LnParams& p, int act, hipStream_t stream);
+hipError_t launch_ln_bwd_dx(const LnParams& p, const void* dY, hipStream_t stream);
+hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t stream);
+hipError_t launch_swiglu_fwd(const void* x, void* y, int64_t M, int Dh, int dtype, hipStream_t stream);
+hipError_t launch_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t M, int Dh, int dtype, hipStream_t stream);
+
+int ln_padded_k(int K);                 // padded K of the kernels, 0 if K is unsupported
+int ln_row_ranges(int64_t M, int N);    // R for the weight-gradient partials
+
+}  // namespace mf

@@ -1,0 +1,171 @@
+// Element-type dispatch, weight preparation and the stand-alone SwiGLU kernels of the
+// LayerNorm->Linear family (the GEMM kernels live in lnlinear_impl.h, one translation unit per type).
+#include "lnlinear_impl.h"
+
+namespace mf {
+
+template <typename T> hipError_t ln_fwd_dispatch(const LnParams& p, int act, hipStream_t stream);
+template <typename T> hipError_t ln_dx_dispatch(const LnParams& p, const void* dY, hipStream_t stream);
+template <typename T> hipError_t ln_dw_dispatch(const LnParams& p, const void* dY, hipStream_t stream);
+extern template hipError_t ln_fwd_dispatch<bf16_t>(const LnParams&, int, hipStream_t);
+extern template hipError_t ln_fwd_dispatch<f16_t>(const LnParams&, int, hipStream_t);
+extern template hipError_t ln_fwd_dispatch<float>(const LnParams&, int, hipStream_t);
+extern template hipError_t ln_dx_dispatch<bf16_t>(const LnParams&, const void*, hipStream_t);
+extern template hipError_t ln_dx_dispatch<f16_t>(const LnParams&, const void*, hipStream_t);
+extern template hipError_t ln_dx_dispatch<float>(const LnParams&, const void*, hipStream_t);
+extern template hipError_t ln_dw_dispatch<bf16_t>(const LnParams&, const void*, hipStream_t);
+extern template hipError_t ln_dw_dispatch<f16_t>(const LnParams&, const void*, hipStream_t);
+extern template hipError_t ln_dw_dispatch<float>(const LnParams&, const void*, hipStream_t);
+
+hipError_t launch_ln_fwd(const LnParams& p, int act, hipStream_t stream) {
+  switch (p.dtype) {
+    case MF_BF16: return ln_fwd_dispatch<bf16_t>(p, act, stream);
+    case MF_F16: return ln_fwd_dispatch<f16_t>(p, act, stream);
+    case MF_F32: return ln_fwd_dispatch<float>(p, act, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_ln_bwd_dx(const LnParams& p, const void* dY, hipStream_t stream) {
+  switch (p.dtype) {
+    case MF_BF16: return ln_dx_dispatch<bf16_t>(p, dY, stream);
+    case MF_F16: return ln_dx_dispatch<f16_t>(p, dY, stream);
+    case MF_F32: return ln_dx_dispatch<float>(p, dY, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t stream) {
+  switch (p.dtype) {
+    case MF_BF16: return ln_dw_dispatch<bf16_t>(p, dY, stream);
+    case MF_F16: return ln_dw_dispatch<f16_t>(p, dY, stream);
+    case MF_F32: return ln_dw_dispatch<float>(p, dY, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// =================================================================================================
+// weight preparation
+// =================================================================================================
+template <typename T>
+__global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= p.N) return;
+  const T* W = reinterpret_cast<const T*>(p.W);
+  const T* gamma = reinterpret_cast<const T*>(p.gamma);
+  const T* beta = reinterpret_cast<const T*>(p.beta);
+  T* Wt = reinterpret_cast<T*>(p.Wt);
+  T* Wg = reinterpret_cast<T*>(p.Wg);
+  float cs = 0.0f, bp = 0.0f;
+  for (int k = 0; k < p.K; ++k) {
+    const float w = to_f(W[(int64_t)k * p.N + n]);
+    const T gw = (T)(to_f(gamma[k]) * w);
+    if (Wt) Wt[(int64_t)n * p.KP + k] = gw;
+    if (Wg) Wg[(int64_t)k * p.N + n] = gw;
+    cs += to_f(gw);
+    if (beta) bp += to_f(beta[k]) * w;
+  }
+  if (Wt)
+    for (int k = p.K; k < p.KP; ++k) Wt[(int64_t)n * p.KP + k] = (T)0.0f;
+  if (p.colsum) p.colsum[n] = cs;
+  if (p.bprime) p.bprime[n] = bp + (p.b ? to_f(reinterpret_cast<const T*>(p.b)[n]) : 0.0f);
+}
+
+hipError_t launch_ln_prep(const LnParams& p, bool forward, hipStream_t stream) {
+  (void)forward;
+  const unsigned blocks = (unsigned)((p.N + 255) / 256);
+  switch (p.dtype) {
+    case MF_BF16: hipLaunchKernelGGL(ln_prep_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    case MF_F16: hipLaunchKernelGGL(ln_prep_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    case MF_F32: hipLaunchKernelGGL(ln_prep_kernel<float>, dim3(blocks), dim3(256), 0, stream, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+int ln_padded_k(int K) {
+  if (K <= 0 || K % 8 != 0) return 0;
+  for (int kp = 16; kp <= 256; kp *= 2)
+    if (K <= kp) return kp;
+  return 0;
+}
+
+int ln_row_ranges(int64_t M, int N) {
+  // about two work-groups per compute unit over (ranges x column blocks); each range at least 256 rows
+  int64_t r = 128;
+  while (r > 1 && M / r < 256) r /= 2;
+  (void)N;
+  return (int)r;
+}
+
+// =================================================================================================
+// stand-alone SwiGLU (fused_transition.py:11-52)
+// =================================================================================================
+template <typename T>
+__global__ void __launch_bounds__(256) swiglu_fwd_kernel(const T* __restrict__ xin, T* __restrict__ y, int64_t M, int Dh) {
+  const int cpr = Dh / 8;
+  const int64_t total = M * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    const frag_t<T> a = ld8<T>(xin + m * 2 * Dh + c);
+    const frag_t<T> gt = ld8<T>(xin + m * 2 * Dh + Dh + c);
+    float h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float gv = to_f(gt[e]); h[e] = gv * sigmoidf_fast(gv) * to_f(a[e]); }
+    st8<T>(y + m * Dh + c, cvt8<T>(h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]));
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) swiglu_bwd_kernel(const T* __restrict__ dy, const T* xin, T* dxo, int64_t M, int Dh) {
+  const int cpr = Dh / 8;
+  const int64_t total = M * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    const frag_t<T> a = ld8<T>(xin + m * 2 * Dh + c);
+    const frag_t<T> gt = ld8<T>(xin + m * 2 * Dh + Dh + c);
+    const frag_t<T> d = ld8<T>(dy + m * Dh + c);
+    float da[8], dg[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gv = to_f(gt[e]), dh = to_f(d[e]);
+      const float sg = sigmoidf_fast(gv), silu = gv * sg;
+      da[e] = dh * silu;
+      dg[e] = dh * (silu * (1.0f - sg) + sg) * to_f(a[e]);
+    }
+    st8<T>(dxo + m * 2 * Dh + c, cvt8<T>(da[0], da[1], da[2], da[3], da[4], da[5], da[6], da[7]));
+    st8<T>(dxo + m * 2 * Dh + Dh + c, cvt8<T>(dg[0], dg[1], dg[2], dg[3], dg[4], dg[5], dg[6], dg[7]));
+  }
+}
+
+static unsigned ew_blocks(int64_t total) {
+  int64_t b = (total + 255) / 256;
+  const int64_t cap = 16LL * num_cu();
+  return (unsigned)(b > cap ? cap : (b < 1 ? 1 : b));
+}
+
+hipError_t launch_swiglu_fwd(const void* x, void* y, int64_t M, int Dh, int dtype, hipStream_t stream) {
+  const unsigned blocks = ew_blocks(M * (Dh / 8));
+  switch (dtype) {
+    case MF_BF16: hipLaunchKernelGGL(swiglu_fwd_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)y, M, Dh); break;
+    case MF_F16: hipLaunchKernelGGL(swiglu_fwd_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, (const f16_t*)x, (f16_t*)y, M, Dh); break;
+    case MF_F32: hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, (float*)y, M, Dh); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t M, int Dh, int dtype, hipStream_t stream) {
+  const unsigned blocks = ew_blocks(M * (Dh / 8));
+  switch (dtype) {
+    case MF_BF16: hipLaunchKernelGGL(swiglu_bwd_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)dy, (const bf16_t*)x, (bf16_t*)dx, M, Dh); break;
+    case MF_F16: hipLaunchKernelGGL(swiglu_bwd_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, (const f16_t*)dy, (const f16_t*)x, (f16_t*)dx, M, Dh); break;
+    case MF_F32: hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)dy, (const float*)x, (float*)dx, M, Dh); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace mf

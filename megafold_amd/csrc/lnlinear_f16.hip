@@ -1,0 +1,7 @@
+// LayerNorm->Linear GEMM kernels instantiated for one element type.
+#include "lnlinear_impl.h"
+namespace mf {
+template hipError_t ln_fwd_dispatch<f16_t>(const LnParams&, int, hipStream_t);
+template hipError_t ln_dx_dispatch<f16_t>(const LnParams&, const void*, hipStream_t);
+template hipError_t ln_dw_dispatch<f16_t>(const LnParams&, const void*, hipStream_t);
+}  // namespace mf

@@ -1,0 +1,685 @@
+// LayerNorm -> Linear (and LayerNorm -> SwiGLU) for gfx950.
+//
+//   mu, r = mean(x), 1/sqrt(var(x) + eps)      x_hat = (x - mu) r      y = x_hat * gamma + beta
+//   out = y W + b                                (reference: fused_layernorm_linear.py:109-218)
+//
+// Forward.  With W' = gamma (.) W (rows scaled),  cs[n] = sum_k W'[k, n]  and
+// b'[n] = sum_k beta[k] W[k, n] + b[n]:
+//       out[m, n] = r[m] * (x[m, :] W'[:, n]) - r[m] mu[m] cs[n] + b'[n]
+// so the MFMA runs on the RAW 16-bit x (no rounding of the normalised activations, no vector-ALU
+// work per input element) and LayerNorm becomes two fused multiply-adds per OUTPUT element.  The row
+// statistics are computed while the x tile is staged into LDS (two-pass variance, fp32) — the
+// "prologue" of the GEMM — and saved as fp32 for the backward.  Each wavefront keeps its slice of
+// W'^T in registers for the whole kernel and walks over row blocks (persistent work-groups), so the
+// only streams are x in and out out.  The SwiGLU variant gives a wavefront matching value/gate
+// column tiles and writes only h = silu(gate) * value.
+//
+// Backward (fused_layernorm_linear.py:226-348, closed forms at 281-306, 345), two kernels, no atomics:
+//   dx:  w = dOut W'^T (contraction over N on the MFMA, W' chunks through LDS, dOut straight from
+//        global), then c1 = mean(x_hat w), c2 = mean(w), dx = (w - x_hat c1 - c2) r in registers: a
+//        lane owns one row, so the two means are register sums plus one lane exchange.
+//   dW:  G = x_hat^T dOut and s = colsum(dOut) per row range (contraction over the rows: both
+//        operands are staged row-major and reach the MFMA through transposing LDS reads), then a small
+//        kernel sums the ranges in a fixed order and forms
+//        dW = gamma G + beta s,  dgamma = rowsum(W (.) G),  dbeta = W s,  db = s.
+#pragma once
+#include "common.h"
+#include "lnlinear.h"
+
+namespace mf {
+
+template <typename T> __device__ __forceinline__ float to_f(T v) { return (float)v; }
+
+// =================================================================================================
+// forward
+// =================================================================================================
+template <typename T, int KP> struct LnLayout {
+  static constexpr int UNIT = 16 / (int)sizeof(T);
+  static constexpr int XSTR = ((KP / UNIT) % 2 == 0) ? KP + UNIT : KP;
+};
+
+__device__ __forceinline__ float sigmoidf_fast(float g) {
+  return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-g * MF_LOG2E));
+}
+
+// Column of W handled by A-operand row m of tile t (see the layout note in common.h): the
+// accumulator of lane half g then holds TILES*16 contiguous columns.
+template <int NTW, int ACT> __device__ __forceinline__ int ln_col(int t, int gm, int rr, int base, int Nhalf) {
+  if (ACT == LN_ACT_NONE) return base + (NTW * 16) * gm + 16 * t + rr;
+  constexpr int TH = NTW / 2;
+  const int th = t % TH, half = t / TH;
+  return half * Nhalf + base + (TH * 16) * gm + 16 * th + rr;
+}
+
+template <int NTW, int ACT> __device__ __forceinline__ bool ln_col_ok(int t, int gm, int rr, int base, int N, int Nhalf) {
+  if (ACT == LN_ACT_NONE) return base + (NTW * 16) * gm + 16 * t + rr < N;
+  constexpr int TH = NTW / 2;
+  return base + (TH * 16) * gm + 16 * (t % TH) + rr < Nhalf;
+}
+
+template <typename T, int KP, int NTW, int ACT, int WN>
+__global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
+  using L = LnLayout<T, KP>;
+  using frag = frag_t<T>;
+  constexpr int KS = KP / 16, CPR = KP / 8;
+  constexpr int TH = NTW / 2;
+  constexpr int OUTW = (ACT == LN_ACT_NONE) ? NTW * 32 : TH * 32;   // output columns per wavefront
+  constexpr int WR = 4 / WN, RB = 32 * WR;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* Xs = reinterpret_cast<T*>(smem_raw);                          // [2][RB][XSTR]
+  float* meanL = reinterpret_cast<float*>(Xs + 2 * RB * L::XSTR);  // [2][RB]
+  float* rstdL = meanL + 2 * RB;                                   // [2][RB]
+  float* csL = rstdL + 2 * RB;                                     // [4 * NTW * 32]
+  float* bpL = csL + 4 * NTW * 32;
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const int wn = w % WN, wr = w / WN;
+  const int Nhalf = p.N / 2;
+  const int NOUT = (ACT == LN_ACT_NONE) ? p.N : Nhalf;             // width of the output / dout
+  const int base = (blockIdx.y * WN + wn) * OUTW;                  // first output column of this wavefront
+  const T* Wt = reinterpret_cast<const T*>(p.Wt);
+  const T* X = reinterpret_cast<const T*>(p.x);
+
+  // ---- this wavefront's slice of W'^T, resident in registers -----------------------------------
+  frag af[NTW][KS];
+  {
+    const int gm = (x >> 2) & 1, rr = 4 * (x >> 3) + (x & 3);
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      const int col = ln_col<NTW, ACT>(t, gm, rr, base, Nhalf);
+      const bool ok = ln_col_ok<NTW, ACT>(t, gm, rr, base, p.N, Nhalf);
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        af[t][s] = ok ? ld8<T>(Wt + (int64_t)col * KP + (KP / 2) * g + 8 * s) : frag_zero<T>();
+    }
+  }
+  // column constants of the work-group's columns: index ((wn * NTW + t) * 2 + g) * 16 + rr
+  for (int i = tid; i < WN * NTW * 32; i += 256) {
+    const int rr = i & 15, gg = (i >> 4) & 1, t = (i >> 5) % NTW, wn2 = (i >> 5) / NTW;
+    const int b2 = (blockIdx.y * WN + wn2) * OUTW;
+    const int col = ln_col<NTW, ACT>(t, gg, rr, b2, Nhalf);
+    const bool ok = ln_col_ok<NTW, ACT>(t, gg, rr, b2, p.N, Nhalf);
+    csL[i] = ok ? p.colsum[col] : 0.0f;
+    bpL[i] = ok ? p.bprime[col] : 0.0f;
+  }
+
+  // ---- staging of one block of rows: x -> LDS, statistics on the way ---------------------------
+  constexpr int items = RB * CPR;
+  constexpr int PFMAX = (items + 255) / 256;
+  frag xr[PFMAX];
+  auto fetch = [&](int64_t rb) {
+#pragma unroll
+    for (int i = 0; i < PFMAX; ++i) {
+      const int item = tid + 256 * i;
+      xr[i] = frag_zero<T>();
+      if (item < items) {
+        const int row = item / CPR, dc = item % CPR;
+        const int64_t m = rb * RB + row;
+        if (m < p.M && 8 * dc < p.K) xr[i] = ld8<T>(X + m * p.K + 8 * dc);
+      }
+    }
+  };
+  auto stash = [&](int64_t rb, int buf) {
+    T* xd = Xs + buf * RB * L::XSTR;
+#pragma unroll
+    for (int i = 0; i < PFMAX; ++i) {
+      const int item = tid + 256 * i;
+      if (item < items) {
+        const int row = item / CPR, dc = item % CPR;
+        st8<T>(xd + row * L::XSTR + 8 * dc, xr[i]);
+        float s = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += to_f(xr[i][e]);
+#pragma unroll
+        for (int msk = 1; msk < CPR; msk <<= 1) s += __shfl_xor(s, msk);
+        const float mu = s / (float)p.K;
+        float d = 0.0f;
+        if (8 * dc < p.K) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { const float c = to_f(xr[i][e]) - mu; d += c * c; }
+        }
+#pragma unroll
+        for (int msk = 1; msk < CPR; msk <<= 1) d += __shfl_xor(d, msk);
+        const float rs = __builtin_amdgcn_rsqf(d / (float)p.K + p.eps);
+        if (dc == 0) {
+          meanL[buf * RB + row] = mu;
+          rstdL[buf * RB + row] = rs;
+          const int64_t m = rb * RB + row;
+          if (ACT != LN_ACT_SWIGLU_BWD && blockIdx.y == 0 && m < p.M) { p.mean[m] = mu; p.rstd[m] = rs; }
+        }
+      }
+    }
+  };
+
+  const int64_t nrb = (p.M + RB - 1) / RB;
+  int64_t rb = blockIdx.x;
+  if (rb < nrb) fetch(rb);
+  int it = 0;
+  for (; rb < nrb; rb += gridDim.x, ++it) {
+    const int buf = it & 1;
+    stash(rb, buf);
+    __syncthreads();
+    if (rb + gridDim.x < nrb) fetch(rb + gridDim.x);
+
+    const T* xt = Xs + buf * RB * L::XSTR + (wr * 32 + x) * L::XSTR;
+    f32x16 acc[NTW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) acc[t] = acc_zero();
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const frag bf = ld8<T>(xt + (KP / 2) * g + 8 * s);
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) acc[t] = mma(af[t][s], bf, acc[t]);
+    }
+
+    const int64_t m = rb * RB + wr * 32 + x;
+    const float mu = meanL[buf * RB + wr * 32 + x], rs = rstdL[buf * RB + wr * 32 + x];
+    const float c0 = -rs * mu;
+    const float* csw = csL + (wn * NTW) * 32 + 16 * g;
+    const float* bpw = bpL + (wn * NTW) * 32 + 16 * g;
+    if (ACT == LN_ACT_NONE) {
+      T* orow = reinterpret_cast<T*>(p.out) + m * p.N;
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        float v[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          v[r] = __builtin_fmaf(acc[t][r], rs, __builtin_fmaf(c0, csw[t * 32 + r], bpw[t * 32 + r]));
+        const int col0 = base + (NTW * 16) * g + 16 * t;
+        if (m < p.M) {
+          if (col0 < p.N) st8<T>(orow + col0, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
+          if (col0 + 8 < p.N) st8<T>(orow + col0 + 8, cvt8<T>(v[8], v[9], v[10], v[11], v[12], v[13], v[14], v[15]));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int th = 0; th < TH; ++th) {
+        float a[16], gt[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          a[r] = __builtin_fmaf(acc[th][r], rs, __builtin_fmaf(c0, csw[th * 32 + r], bpw[th * 32 + r]));
+          gt[r] = __builtin_fmaf(acc[TH + th][r], rs, __builtin_fmaf(c0, csw[(TH + th) * 32 + r], bpw[(TH + th) * 32 + r]));
+        }
+        const int col0 = base + (TH * 16) * g + 16 * th;   // column of h (and of dh)
+        if (m < p.M && col0 < Nhalf) {
+          const bool two = col0 + 8 < Nhalf;
+          if (ACT == LN_ACT_SWIGLU) {
+            float h[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) h[r] = a[r] * gt[r] * sigmoidf_fast(gt[r]);
+            T* orow = reinterpret_cast<T*>(p.out) + m * Nhalf + col0;
+            st8<T>(orow, cvt8<T>(h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]));
+            if (two) st8<T>(orow + 8, cvt8<T>(h[8], h[9], h[10], h[11], h[12], h[13], h[14], h[15]));
+          } else {
+            // SwiGLU backward on the recomputed pre-activation (fused_transition.py:44-47)
+            const T* drow = reinterpret_cast<const T*>(p.dout) + m * Nhalf + col0;
+            const frag d0 = ld8<T>(drow);
+            const frag d1 = two ? ld8<T>(drow + 8) : frag_zero<T>();
+            float da[16], dg[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float dh = to_f(r < 8 ? d0[r & 7] : d1[r & 7]);
+              const float sg = sigmoidf_fast(gt[r]);
+              const float silu = gt[r] * sg;
+              da[r] = dh * silu;
+              dg[r] = dh * a[r] * (sg + silu * (1.0f - sg));
+            }
+            T* urow = reinterpret_cast<T*>(p.du) + m * p.N;
+            st8<T>(urow + col0, cvt8<T>(da[0], da[1], da[2], da[3], da[4], da[5], da[6], da[7]));
+            st8<T>(urow + Nhalf + col0, cvt8<T>(dg[0], dg[1], dg[2], dg[3], dg[4], dg[5], dg[6], dg[7]));
+            if (two) {
+              st8<T>(urow + col0 + 8, cvt8<T>(da[8], da[9], da[10], da[11], da[12], da[13], da[14], da[15]));
+              st8<T>(urow + Nhalf + col0 + 8, cvt8<T>(dg[8], dg[9], dg[10], dg[11], dg[12], dg[13], dg[14], dg[15]));
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+static int g_num_cu = 0;
+static inline int num_cu() {
+  if (g_num_cu == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_num_cu = n;
+    else
+      g_num_cu = 256;
+  }
+  return g_num_cu;
+}
+
+template <typename T, int KP, int NTW, int ACT, int WN>
+static hipError_t launch_fwd_w(const LnParams& p, hipStream_t stream) {
+  using L = LnLayout<T, KP>;
+  constexpr int OUTW = (ACT == LN_ACT_NONE) ? NTW * 32 : (NTW / 2) * 32;
+  constexpr int RB = 32 * (4 / WN);
+  const int NOUT = (ACT == LN_ACT_NONE) ? p.N : p.N / 2;
+  const int gy = (NOUT + WN * OUTW - 1) / (WN * OUTW);
+  const int64_t nrb = (p.M + RB - 1) / RB;
+  int64_t gx = 2LL * num_cu() / gy;
+  if (gx < 1) gx = 1;
+  if (gx > nrb) gx = nrb;
+  const size_t smem = (size_t)2 * RB * L::XSTR * sizeof(T) + (size_t)4 * RB * 4 + (size_t)2 * 4 * NTW * 32 * 4;
+  auto kern = ln_fwd_kernel<T, KP, NTW, ACT, WN>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)gx, (unsigned)gy), dim3(256), smem, stream, p);
+  return hipGetLastError();
+}
+
+// Tiles per wavefront (NTW) and wavefronts along the columns (WN) by output width; the remaining
+// wavefronts of the work-group take further 32-row blocks.
+template <typename T, int KP, int ACT> static hipError_t launch_fwd_k(const LnParams& p, hipStream_t stream) {
+  const int NOUT = (ACT == LN_ACT_NONE) ? p.N : p.N / 2;
+  constexpr bool wide = sizeof(T) == 4 || KP > 128;   // fragments twice as large: halve the resident slice
+  if constexpr (ACT == LN_ACT_NONE) {
+    if (NOUT <= 32) return launch_fwd_w<T, KP, 1, ACT, 1>(p, stream);
+    if (NOUT <= 128) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
+    if (NOUT <= 256 || wide) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
+    return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
+  } else {
+    if (NOUT <= 64) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
+    if (NOUT <= 128 || wide) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
+    return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
+  }
+}
+
+template <typename T, int KP> static hipError_t launch_fwd_a(const LnParams& p, int act, hipStream_t stream) {
+  switch (act) {
+    case LN_ACT_NONE: return launch_fwd_k<T, KP, LN_ACT_NONE>(p, stream);
+    case LN_ACT_SWIGLU: return launch_fwd_k<T, KP, LN_ACT_SWIGLU>(p, stream);
+    case LN_ACT_SWIGLU_BWD: return launch_fwd_k<T, KP, LN_ACT_SWIGLU_BWD>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <typename T> hipError_t ln_fwd_dispatch(const LnParams& p, int act, hipStream_t stream) {
+  switch (p.KP) {
+    case 16: return launch_fwd_a<T, 16>(p, act, stream);
+    case 32: return launch_fwd_a<T, 32>(p, act, stream);
+    case 64: return launch_fwd_a<T, 64>(p, act, stream);
+    case 128: return launch_fwd_a<T, 128>(p, act, stream);
+    case 256: return launch_fwd_a<T, 256>(p, act, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+
+
+
+// =================================================================================================
+// backward: dx
+// =================================================================================================
+template <typename T, int KP>
+__global__ void __launch_bounds__(256, 2) ln_bwd_dx_kernel(const LnParams p, const T* __restrict__ dY) {
+  using frag = frag_t<T>;
+  constexpr int KPT = KP < 32 ? 32 : KP;       // rows of the W' operand, padded to whole tiles
+  constexpr int KT = KPT / 32;
+  constexpr int NC = 64;                       // columns of N per staged chunk
+  constexpr int UNIT = 16 / (int)sizeof(T);
+  constexpr int WSTR = ((NC / UNIT) % 2 == 0) ? NC + UNIT : NC;
+  constexpr int PF = (KPT * (NC / 8) + 255) / 256;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* Ws = reinterpret_cast<T*>(smem_raw);      // [2][KPT][WSTR]
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const T* Wg = reinterpret_cast<const T*>(p.Wg);
+  const T* X = reinterpret_cast<const T*>(p.x);
+  T* dX = reinterpret_cast<T*>(p.dx);
+  const int N = p.N, K = p.K;
+  const int nchunks = (N + NC - 1) / NC;
+
+  frag wr_[PF];
+  auto fetch_w = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int item = tid + 256 * i;
+      wr_[i] = frag_zero<T>();
+      if (item < KPT * (NC / 8)) {
+        const int k = item / (NC / 8), nc = item % (NC / 8);
+        const int n = c * NC + 8 * nc;
+        if (k < K && n < N) wr_[i] = ld8<T>(Wg + (int64_t)k * N + n);
+      }
+    }
+  };
+  auto stash_w = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int item = tid + 256 * i;
+      if (item < KPT * (NC / 8)) {
+        const int k = item / (NC / 8), nc = item % (NC / 8);
+        st8<T>(Ws + (buf * KPT + k) * WSTR + 8 * nc, wr_[i]);
+      }
+    }
+  };
+
+  const int64_t nrb = (p.M + 127) / 128;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t m = rb * 128 + w * 32 + x;
+    const int64_t mc = m < p.M ? m : p.M - 1;
+    const T* dyrow = dY + mc * N;
+    f32x16 acc[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) acc[kt] = acc_zero();
+
+    frag yb[4];
+    auto fetch_y = [&](int c) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int n = c * NC + 32 * g + 8 * s;
+        yb[s] = (m < p.M && n < N) ? ld8<T>(dyrow + n) : frag_zero<T>();
+      }
+    };
+    __syncthreads();          // the previous row block is done with both W' buffers
+    fetch_w(0);
+    fetch_y(0);
+    stash_w(0);
+    __syncthreads();
+    for (int c = 0; c < nchunks; ++c) {
+      const int buf = c & 1;
+      frag yc[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) yc[s] = yb[s];
+      const bool more = c + 1 < nchunks;
+      if (more) { fetch_w(c + 1); fetch_y(c + 1); }
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        const T* wrow = Ws + (buf * KPT + dsel<KPT>(kt, x)) * WSTR + 32 * g;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc[kt] = mma(ld8<T>(wrow + 8 * s), yc[s], acc[kt]);
+      }
+      if (more) stash_w(buf ^ 1);
+      __syncthreads();
+    }
+
+    // ---- LayerNorm backward on the row this lane owns: register r of tile kt <-> k = (KPT/2) g + 16 kt + r
+    const float mu = p.mean[mc], rs = p.rstd[mc];
+    float xh[KT][16];
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
+        const frag xv = k0 < K ? ld8<T>(X + mc * K + k0) : frag_zero<T>();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float v = k0 < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
+          xh[kt][8 * u + e] = v;
+          s1 += v * acc[kt][8 * u + e];
+          s2 += acc[kt][8 * u + e];
+        }
+      }
+    }
+    s1 += __shfl_xor(s1, 32);
+    s2 += __shfl_xor(s2, 32);
+    const float c1 = s1 / (float)K, c2 = s2 / (float)K;
+    if (m < p.M) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
+          if (k0 < K) {
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (acc[kt][8 * u + e] - (xh[kt][8 * u + e] * c1 + c2)) * rs;
+            st8<T>(dX + m * K + k0, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
+          }
+        }
+    }
+  }
+}
+
+template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
+  constexpr int KPT = KP < 32 ? 32 : KP;
+  constexpr int UNIT = 16 / (int)sizeof(T);
+  constexpr int WSTR = ((64 / UNIT) % 2 == 0) ? 64 + UNIT : 64;
+  const size_t smem = (size_t)2 * KPT * WSTR * sizeof(T);
+  const int64_t nrb = (p.M + 127) / 128;
+  int64_t gx = 2LL * num_cu();
+  if (gx > nrb) gx = nrb;
+  auto kern = ln_bwd_dx_kernel<T, KP>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)gx), dim3(256), smem, stream, p, reinterpret_cast<const T*>(dY));
+  return hipGetLastError();
+}
+
+template <typename T> hipError_t ln_dx_dispatch(const LnParams& p, const void* dY, hipStream_t stream) {
+  switch (p.KP) {
+    case 16: return launch_dx_t<T, 16>(p, dY, stream);
+    case 32: return launch_dx_t<T, 32>(p, dY, stream);
+    case 64: return launch_dx_t<T, 64>(p, dY, stream);
+    case 128: return launch_dx_t<T, 128>(p, dY, stream);
+    case 256: return launch_dx_t<T, 256>(p, dY, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+
+// =================================================================================================
+// backward: G = x_hat^T dOut, s = colsum(dOut), then dW / dgamma / dbeta / db
+// =================================================================================================
+template <int KP> struct DwShape {
+  static constexpr int KPT = KP < 32 ? 32 : KP;
+  static constexpr int WK = KPT >= 256 ? 4 : (KPT >= 64 ? 2 : 1);   // wavefronts along k
+  static constexpr int KTW = KPT / (32 * WK);                        // k tiles per wavefront
+  static constexpr int WNN = 4 / WK;                                  // wavefronts along n
+  static constexpr int NTW = WNN == 4 ? 1 : 2;                        // n tiles per wavefront
+  static constexpr int CW = WNN * NTW * 32;                           // columns per work-group
+};
+
+template <typename T, int KP>
+__global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, const T* __restrict__ dY) {
+  using frag = frag_t<T>;
+  using Sh = DwShape<KP>;
+  constexpr int KPT = Sh::KPT, KTW = Sh::KTW, WNN = Sh::WNN, NTW = Sh::NTW, CW = Sh::CW;
+  constexpr int RT = 64;                       // rows per staged tile
+  constexpr int UNIT = 16 / (int)sizeof(T);
+  constexpr int XSTR = ((KPT / UNIT) % 2 == 0) ? KPT + UNIT : KPT;
+  constexpr int YSTR = ((CW / UNIT) % 2 == 0) ? CW + UNIT : CW;
+  constexpr int XI = RT * (KPT / 8), YI = RT * (CW / 8);
+  constexpr int PFX = (XI + 255) / 256, PFY = (YI + 255) / 256;
+  static_assert(256 % (CW / 8) == 0, "a thread must keep one column chunk");
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* Xs = reinterpret_cast<T*>(smem_raw);      // [2][RT][XSTR]  normalised rows
+  T* Ys = Xs + 2 * RT * XSTR;                  // [2][RT][YSTR]
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const int wk = w / WNN, wn = w % WNN;
+  const int range = blockIdx.x, cb = blockIdx.y * CW;
+  const int64_t m_begin = (int64_t)range * p.rows_per_range;
+  const int64_t m_end = m_begin + p.rows_per_range < p.M ? m_begin + p.rows_per_range : p.M;
+  const T* X = reinterpret_cast<const T*>(p.x);
+  const int K = p.K, N = p.N;
+
+  f32x16 acc[KTW][NTW];
+#pragma unroll
+  for (int a = 0; a < KTW; ++a)
+#pragma unroll
+    for (int b = 0; b < NTW; ++b) acc[a][b] = acc_zero();
+  float colsum[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) colsum[e] = 0.0f;
+
+  frag xr[PFX], yr[PFY];
+  float mur[PFX], rsr[PFX];
+  auto fetch = [&](int64_t m0) {
+#pragma unroll
+    for (int i = 0; i < PFX; ++i) {
+      const int item = tid + 256 * i;
+      xr[i] = frag_zero<T>(); mur[i] = 0.0f; rsr[i] = 0.0f;
+      if (item < XI) {
+        const int row = item / (KPT / 8), dc = item % (KPT / 8);
+        const int64_t m = m0 + row;
+        if (m < m_end && 8 * dc < K) { xr[i] = ld8<T>(X + m * K + 8 * dc); mur[i] = p.mean[m]; rsr[i] = p.rstd[m]; }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PFY; ++i) {
+      const int item = tid + 256 * i;
+      yr[i] = frag_zero<T>();
+      if (item < YI) {
+        const int row = item / (CW / 8), cc = item % (CW / 8);
+        const int64_t m = m0 + row;
+        const int n = cb + 8 * cc;
+        if (m < m_end && n < N) yr[i] = ld8<T>(dY + m * N + n);
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PFX; ++i) {
+      const int item = tid + 256 * i;
+      if (item < XI) {
+        const int row = item / (KPT / 8), dc = item % (KPT / 8);
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (to_f(xr[i][e]) - mur[i]) * rsr[i];   // rows past the end: rs = 0
+        st8<T>(Xs + (buf * RT + row) * XSTR + 8 * dc, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PFY; ++i) {
+      const int item = tid + 256 * i;
+      if (item < YI) {
+        const int row = item / (CW / 8), cc = item % (CW / 8);
+        st8<T>(Ys + (buf * RT + row) * YSTR + 8 * cc, yr[i]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) colsum[e] += to_f(yr[i][e]);
+      }
+    }
+  };
+
+  if (m_begin < m_end) fetch(m_begin);
+  int it = 0;
+  for (int64_t m0 = m_begin; m0 < m_end; m0 += RT, ++it) {
+    const int buf = it & 1;
+    stash(buf);
+    __syncthreads();
+    if (m0 + RT < m_end) fetch(m0 + RT);
+    const T* xs = Xs + buf * RT * XSTR;
+    const T* ys = Ys + buf * RT * YSTR;
+#pragma unroll
+    for (int st = 0; st < RT / 16; ++st) {
+      frag bf[NTW];
+#pragma unroll
+      for (int b = 0; b < NTW; ++b) {
+        const int nb = (wn * NTW + b) * 32;
+        bf[b] = TrRead<T>::read(ys, YSTR, 16 * st, g, l, nb + plain_chunk(l), nb + x);
+      }
+#pragma unroll
+      for (int a = 0; a < KTW; ++a) {
+        const int kb = (wk * KTW + a) * 32;
+        const frag af = TrRead<T>::read(xs, XSTR, 16 * st, g, l, kb + plain_chunk(l), kb + x);
+#pragma unroll
+        for (int b = 0; b < NTW; ++b) acc[a][b] = mma(af, bf[b], acc[a][b]);
+      }
+    }
+  }
+
+  // ---- partial G: natural accumulator layout, lane = column n, registers = rows k ----------------
+  float* Gp = p.Gpart + (int64_t)range * K * N;
+#pragma unroll
+  for (int a = 0; a < KTW; ++a)
+#pragma unroll
+    for (int b = 0; b < NTW; ++b) {
+      const int n = cb + (wn * NTW + b) * 32 + x;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int k = (wk * KTW + a) * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (k < K && n < N) Gp[(int64_t)k * N + n] = acc[a][b][r];
+      }
+    }
+  // ---- partial column sums: threads with the same column chunk are 256 / (CW/8) apart ------------
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem_raw);       // [256][8]
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[tid * 8 + e] = colsum[e];
+  __syncthreads();
+  if (tid < CW) {
+    const int cc = tid / 8, e = tid % 8;
+    float s = 0.0f;
+    for (int j = cc; j < 256; j += CW / 8) s += red[j * 8 + e];
+    const int n = cb + tid;
+    if (n < N) p.spart[(int64_t)range * N + n] = s;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) {
+  const int k = blockIdx.x, tid = threadIdx.x;
+  const T* W = reinterpret_cast<const T*>(p.W);
+  const float gam = to_f(reinterpret_cast<const T*>(p.gamma)[k]);
+  const float bet = p.beta ? to_f(reinterpret_cast<const T*>(p.beta)[k]) : 0.0f;
+  float dg = 0.0f, dbt = 0.0f;
+  for (int n = tid; n < p.N; n += 256) {
+    float G = 0.0f, s = 0.0f;
+    for (int r = 0; r < p.R; ++r) {
+      G += p.Gpart[((int64_t)r * p.K + k) * p.N + n];
+      s += p.spart[(int64_t)r * p.N + n];
+    }
+    const float wv = to_f(W[(int64_t)k * p.N + n]);
+    p.dW[(int64_t)k * p.N + n] = gam * G + bet * s;
+    dg += wv * G;
+    dbt += wv * s;
+    if (k == 0 && p.db) p.db[n] = s;
+  }
+  __shared__ float r1[256], r2[256];
+  r1[tid] = dg; r2[tid] = dbt;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (tid < o) { r1[tid] += r1[tid + o]; r2[tid] += r2[tid + o]; }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    p.dgamma[k] = r1[0];
+    if (p.dbeta) p.dbeta[k] = r2[0];
+  }
+}
+
+
+template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, const void* dY, hipStream_t stream) {
+  using Sh = DwShape<KP>;
+  constexpr int UNIT = 16 / (int)sizeof(T);
+  constexpr int XSTR = ((Sh::KPT / UNIT) % 2 == 0) ? Sh::KPT + UNIT : Sh::KPT;
+  constexpr int YSTR = ((Sh::CW / UNIT) % 2 == 0) ? Sh::CW + UNIT : Sh::CW;
+  size_t smem = (size_t)2 * 64 * (XSTR + YSTR) * sizeof(T);
+  if (smem < 256 * 8 * 4) smem = 256 * 8 * 4;
+  const int gy = (p.N + Sh::CW - 1) / Sh::CW;
+  auto kern = ln_bwd_dw_kernel<T, KP>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)p.R, (unsigned)gy), dim3(256), smem, stream, p, reinterpret_cast<const T*>(dY));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ln_bwd_finalize_kernel<T>, dim3((unsigned)p.K), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T> hipError_t ln_dw_dispatch(const LnParams& p, const void* dY, hipStream_t stream) {
+  switch (p.KP) {
+    case 16: return launch_dw_t<T, 16>(p, dY, stream);
+    case 32: return launch_dw_t<T, 32>(p, dY, stream);
+    case 64: return launch_dw_t<T, 64>(p, dY, stream);
+    case 128: return launch_dw_t<T, 128>(p, dY, stream);
+    case 256: return launch_dw_t<T, 256>(p, dY, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+
+}  // namespace mf

@@ -1,0 +1,200 @@
+"""Fused LayerNorm -> Linear on MI355X.
+
+Drop-in for the reference module ``megafold/model/FusedLayernormLinear/fused_layernorm_linear.py``:
+the ``LayernormLinear`` module (fused_layernorm_linear.py:498-545), ``LayernormLinearFunction``
+(:477-495) and the host functions ``layernorm_linear_forward`` / ``layernorm_linear_backward``
+(:351-405, :408-474), with the same parameter names (``WEIGHT``, ``BIAS``, ``linear_weight`` stored
+``[K, N]``, ``linear_bias``), the same initialisation and the same autocast contract
+(``custom_fwd(cast_inputs=torch.bfloat16)``).  The work is done by HIP kernels reached through
+``mf_lnlinear_fwd`` / ``mf_lnlinear_bwd``.
+
+Differences from the reference, all on purpose:
+
+* Row statistics are kept in fp32 (the reference stores them in the input dtype, :361-362).
+* No atomics: dW, dgamma, dbeta and the linear-bias gradient come from fixed-order reductions.
+* Every shape with K a multiple of 8 (K <= 256) and N a multiple of 8 takes the fused path; the
+  reference only fuses shapes found in its tuning tables (helper.py) and silently runs eager PyTorch
+  otherwise (:539-541).  Shapes outside the kernels' range run the same eager GPU expression here.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ... import _lib
+
+__all__ = ["LayernormLinear", "LayernormLinearFunction", "layernorm_linear_forward", "layernorm_linear_backward",
+           "fused_shape_supported"]
+
+EPS = 1e-5  # literal in the reference launch (fused_layernorm_linear.py:368)
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def fused_shape_supported(K: int, N: int, dtype, act: int = _lib.MF_ACT_NONE) -> bool:
+    mult = 16 if act == _lib.MF_ACT_SWIGLU else 8
+    return dtype in _FLOATS and K % 8 == 0 and 0 < K <= 256 and N > 0 and N % mult == 0
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def _args(a2d, b, linear_bias, WEIGHT, BIAS, act, stream_dev):
+    M, K = a2d.shape
+    a = _lib.LnLinearArgs()
+    a.M, a.K, a.N = M, K, b.shape[1]
+    a.dtype = _lib.dtype_code(a2d.dtype)
+    a.act = act
+    a.eps = EPS
+    a.x, a.gamma, a.beta, a.W, a.b = _ptr(a2d), _ptr(WEIGHT), _ptr(BIAS), _ptr(b), _ptr(linear_bias)
+    a.stream = torch.cuda.current_stream(stream_dev).cuda_stream
+    return a
+
+
+def _same_dtype(ref, *ts):
+    return [None if t is None else (t if t.dtype == ref.dtype else t.to(ref.dtype)).contiguous() for t in ts]
+
+
+def layernorm_linear_forward(a, b, linear_bias, WEIGHT, BIAS, has_layernorm_bias=True, has_linear_bias=False,
+                             forward_config=None, act=_lib.MF_ACT_NONE):
+    """Returns ``(c, a2d, b, Mean, RSTD)`` like the reference (fused_layernorm_linear.py:351-405); Mean and
+    RSTD are fp32.  ``forward_config`` (a Triton tile table entry in the reference) is ignored."""
+    shape = a.shape
+    a2d = a.reshape(-1, shape[-1])
+    assert a2d.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert a2d.is_contiguous(), "Matrix A must be contiguous"
+    if not a2d.is_cuda:
+        raise RuntimeError("LayernormLinear runs on the GPU only (got device %s)" % a2d.device)
+    M, K = a2d.shape
+    N = b.shape[1]
+    b, linear_bias, WEIGHT, BIAS = _same_dtype(a2d, b, linear_bias if has_linear_bias else None, WEIGHT,
+                                               BIAS if has_layernorm_bias else None)
+    lib = _lib.lib()
+    n_out = N // 2 if act == _lib.MF_ACT_SWIGLU else N
+    with torch.cuda.device(a2d.device):
+        c = torch.empty((M, n_out), dtype=a2d.dtype, device=a2d.device)
+        Mean = torch.empty((M,), dtype=torch.float32, device=a2d.device)
+        RSTD = torch.empty((M,), dtype=torch.float32, device=a2d.device)
+        args = _args(a2d, b, linear_bias, WEIGHT, BIAS, act, a2d.device)
+        args.out, args.mean, args.rstd = c.data_ptr(), Mean.data_ptr(), RSTD.data_ptr()
+        nbytes = lib.mf_lnlinear_fwd_workspace_bytes(C.byref(args))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=a2d.device)
+        args.workspace, args.workspace_bytes = ws.data_ptr(), nbytes
+        _lib.check(lib.mf_lnlinear_fwd(C.byref(args)), "mf_lnlinear_fwd")
+    return c.view(shape[:-1] + (n_out,)), a2d, b, Mean, RSTD
+
+
+def layernorm_linear_backward(dOUT, X, B, Mean, RSTD, WEIGHT, BIAS, has_layernorm_bias=True, has_linear_bias=False,
+                              backward_config=None, act=_lib.MF_ACT_NONE):
+    """Returns ``(dX, dB, dLinearBias, dWEIGHT, dBIAS)`` like the reference (fused_layernorm_linear.py:408-474),
+    parameter gradients cast to X's dtype (:470-472)."""
+    dshape = dOUT.shape
+    dOUT = dOUT.reshape(-1, dshape[-1])
+    M, K = X.shape
+    N = B.shape[1]
+    if dOUT.dtype != X.dtype:
+        dOUT = dOUT.to(X.dtype)
+    dOUT = dOUT.contiguous()
+    B, WEIGHT, BIAS = _same_dtype(X, B, WEIGHT, BIAS if has_layernorm_bias else None)
+    lib = _lib.lib()
+    with torch.cuda.device(X.device):
+        dX = torch.empty((M, K), dtype=X.dtype, device=X.device)
+        dB = torch.empty((K, N), dtype=torch.float32, device=X.device)
+        dWEIGHT = torch.empty((K,), dtype=torch.float32, device=X.device)
+        dBIAS = torch.empty((K,), dtype=torch.float32, device=X.device) if has_layernorm_bias else None
+        dLin = torch.empty((N,), dtype=torch.float32, device=X.device) if has_linear_bias else None
+        args = _args(X, B, None, WEIGHT, BIAS, act, X.device)
+        args.mean, args.rstd = Mean.data_ptr(), RSTD.data_ptr()
+        args.dout, args.dx, args.dW = dOUT.data_ptr(), dX.data_ptr(), dB.data_ptr()
+        args.db, args.dgamma, args.dbeta = _ptr(dLin), dWEIGHT.data_ptr(), _ptr(dBIAS)
+        nbytes = lib.mf_lnlinear_bwd_workspace_bytes(C.byref(args))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=X.device)
+        args.workspace, args.workspace_bytes = ws.data_ptr(), nbytes
+        _lib.check(lib.mf_lnlinear_bwd(C.byref(args)), "mf_lnlinear_bwd")
+    dX = dX.view(dshape[:-1] + (K,))
+    dB, dWEIGHT = dB.to(X.dtype), dWEIGHT.to(X.dtype)
+    if dBIAS is not None:
+        dBIAS = dBIAS.to(X.dtype)
+    if dLin is not None:
+        dLin = dLin.to(X.dtype)
+    return dX, dB, dLin, dWEIGHT, dBIAS
+
+
+class LayernormLinearFunction(torch.autograd.Function):
+    """Same contract as the reference class of this name (fused_layernorm_linear.py:477-495)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx, X, linear_weight, linear_bias, WEIGHT, BIAS, has_layernorm_bias=True, has_linear_bias=False,
+                supported_configs=None, act=_lib.MF_ACT_NONE):
+        X = X.contiguous()
+        c, X2, W, Mean, RSTD = layernorm_linear_forward(X, linear_weight, linear_bias, WEIGHT, BIAS, has_layernorm_bias,
+                                                        has_linear_bias, act=act)
+        ctx.save_for_backward(X2, W, Mean, RSTD, WEIGHT, BIAS)
+        ctx.x_shape = X.shape
+        ctx.has_layernorm_bias = has_layernorm_bias
+        ctx.has_linear_bias = has_linear_bias
+        ctx.act = act
+        return c
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dOUT):
+        X, W, Mean, RSTD, WEIGHT, BIAS = ctx.saved_tensors
+        dX, dB, dLin, dWEIGHT, dBIAS = layernorm_linear_backward(dOUT, X, W, Mean, RSTD, WEIGHT, BIAS,
+                                                                 ctx.has_layernorm_bias, ctx.has_linear_bias,
+                                                                 act=ctx.act)
+        return dX.view(ctx.x_shape), dB, dLin, dWEIGHT, dBIAS, None, None, None, None
+
+
+class LayernormLinear(nn.Module):
+    """``LayerNorm(K)`` followed by ``Linear(K, N)``; parameters and initialisation as the reference
+    (fused_layernorm_linear.py:498-534)."""
+
+    def __init__(self, K, N, has_layernorm_bias=True, has_linear_bias=True, device=None, dtype=None):
+        factory_kwargs = {"device": device, "dtype": dtype}
+        super().__init__()
+        self.K = K
+        self.N = N
+        self.has_layernorm_bias = has_layernorm_bias
+        self.has_linear_bias = has_linear_bias
+        self.WEIGHT = nn.Parameter(torch.empty(K, **factory_kwargs))  # LayerNorm weight
+        self.BIAS = nn.Parameter(torch.empty(K, **factory_kwargs)) if has_layernorm_bias else None
+        self.linear_weight = nn.Parameter(torch.empty((K, N), **factory_kwargs))  # nn.Linear.weight transposed
+        self.linear_bias = nn.Parameter(torch.empty((N,), **factory_kwargs)) if has_linear_bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.ones_(self.WEIGHT)
+        if self.has_layernorm_bias:
+            nn.init.zeros_(self.BIAS)
+        # kaiming-uniform of the [N, K] matrix an nn.Linear would hold, stored transposed
+        tmp = torch.empty((self.N, self.K), device=self.linear_weight.device, dtype=self.linear_weight.dtype)
+        with torch.no_grad():
+            nn.init.kaiming_uniform_(tmp, a=math.sqrt(5))
+            self.linear_weight.copy_(tmp.T)
+        if self.has_linear_bias:
+            bound = 1 / math.sqrt(self.K) if self.K > 0 else 0
+            nn.init.uniform_(self.linear_bias, -bound, bound)
+
+    def _eager(self, X):
+        return F.linear(F.layer_norm(X, (self.K,), self.WEIGHT, self.BIAS, EPS), self.linear_weight.T, self.linear_bias)
+
+    def forward(self, X, act=_lib.MF_ACT_NONE):
+        dtype = torch.bfloat16 if torch.is_autocast_enabled() else X.dtype
+        if not fused_shape_supported(self.K, self.N, dtype, act):
+            # same expression the reference falls back to (fused_layernorm_linear.py:541), on the GPU
+            out = self._eager(X)
+            if act == _lib.MF_ACT_SWIGLU:
+                a, g = out.chunk(2, dim=-1)
+                out = F.silu(g) * a
+            return out
+        return LayernormLinearFunction.apply(X, self.linear_weight, self.linear_bias, self.WEIGHT, self.BIAS,
+                                             self.has_layernorm_bias, self.has_linear_bias, None, act)
+
+    def extra_repr(self):
+        return f"K={self.K}, N={self.N}, has_linear_bias={self.has_linear_bias}"

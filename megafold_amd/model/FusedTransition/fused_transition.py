@@ -1,0 +1,128 @@
+"""Fused LayerNorm -> SwiGLU Transition on MI355X.
+
+Drop-in for the reference module ``megafold/model/FusedTransition/fused_transition.py``:
+``FusedTransition`` (fused_transition.py:118-151), ``FusedSwiGLU`` / ``FusedSwiGLUFunction`` (:96-116) and
+the host functions ``swiglu_forward`` / ``swiglu_backward`` (:55-93).  Parameter layout is unchanged
+(``ff.0`` LayernormLinear or LayerNorm/Linear, ``ff.2`` / ``ff.3`` output Linear), so checkpoints load.
+
+``SwiGLU(u) = silu(u[..., d:]) * u[..., :d]`` — the gate is the SECOND half (fused_transition.py:22-24).
+
+With ``include_ln`` and ``use_layernormlinear`` (the form the Pairformer uses) the first three stages
+run as ONE kernel: LayerNorm statistics in the GEMM prologue, SwiGLU in its epilogue, so the
+``[M, 2*dim_inner]`` pre-activation is never written; the backward recomputes it tile by tile.
+The other variants use the stand-alone SwiGLU kernels (``mf_swiglu_fwd`` / ``mf_swiglu_bwd``).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from ... import _lib
+from ..FusedLayernormLinear.fused_layernorm_linear import LayernormLinear
+
+__all__ = ["FusedTransition", "FusedSwiGLU", "FusedSwiGLUFunction", "swiglu_forward", "swiglu_backward"]
+
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def _check(x):
+    if not x.is_cuda:
+        raise RuntimeError("FusedSwiGLU runs on the GPU only (got device %s)" % x.device)
+    if x.dtype not in _FLOATS:
+        raise TypeError("unsupported dtype %s" % x.dtype)
+
+
+def swiglu_forward(x):
+    """x = [left, right] -> (x2d, silu(right) * left), as the reference (fused_transition.py:55-75)."""
+    _check(x)
+    ori_shape = x.shape
+    D = ori_shape[-1]
+    dim_out = D // 2
+    if D % 16 != 0:
+        raise ValueError("SwiGLU needs a last dimension that is a multiple of 16, got %d" % D)
+    x2 = x.reshape(-1, D).contiguous()
+    M = x2.shape[0]
+    with torch.cuda.device(x.device):
+        y = torch.empty((M, dim_out), device=x.device, dtype=x.dtype)
+        rc = _lib.lib().mf_swiglu_fwd(x2.data_ptr(), y.data_ptr(), M, dim_out, _lib.dtype_code(x.dtype),
+                                      torch.cuda.current_stream(x.device).cuda_stream)
+        _lib.check(rc, "mf_swiglu_fwd")
+    return x2, y.view(ori_shape[:-1] + (dim_out,))
+
+
+def swiglu_backward(x, dy):
+    """dy -> [dleft, dright] (fused_transition.py:78-93).  A new tensor is returned; the saved input
+    is not overwritten."""
+    ori_shape = dy.shape
+    D = ori_shape[-1]
+    dy2 = dy.reshape(-1, D)
+    if dy2.dtype != x.dtype:
+        dy2 = dy2.to(x.dtype)
+    dy2 = dy2.contiguous()
+    M = dy2.shape[0]
+    with torch.cuda.device(x.device):
+        dx = torch.empty_like(x)
+        rc = _lib.lib().mf_swiglu_bwd(dy2.data_ptr(), x.data_ptr(), dx.data_ptr(), M, D, _lib.dtype_code(x.dtype),
+                                      torch.cuda.current_stream(x.device).cuda_stream)
+        _lib.check(rc, "mf_swiglu_bwd")
+    return dx.view(ori_shape[:-1] + (D * 2,))
+
+
+class FusedSwiGLUFunction(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx, input):
+        x2, output = swiglu_forward(input)
+        ctx.save_for_backward(x2)
+        ctx.in_shape = input.shape
+        return output
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        (x2,) = ctx.saved_tensors
+        return swiglu_backward(x2, grad_output).view(ctx.in_shape)
+
+
+class FusedSwiGLU(nn.Module):
+    def forward(self, x):
+        return FusedSwiGLUFunction.apply(x)
+
+
+class FusedTransition(nn.Module):
+    def __init__(self, dim, expansion_factor=4, include_ln=True, use_layernormlinear=True, device=None, dtype=None):
+        factory_kwargs = {"device": device, "dtype": dtype}
+        super().__init__()
+        self.dim = dim
+        dim_inner = int(dim * expansion_factor)
+        self.dim_inner = dim_inner
+        self._fused_ln_swiglu = bool(include_ln and use_layernormlinear)
+        if include_ln:
+            if use_layernormlinear:
+                self.ff = nn.Sequential(
+                    LayernormLinear(dim, dim_inner * 2, has_linear_bias=False, **factory_kwargs),
+                    FusedSwiGLU(),
+                    nn.Linear(dim_inner, dim, bias=False, **factory_kwargs),
+                )
+            else:
+                self.ff = nn.Sequential(
+                    nn.LayerNorm(dim, **factory_kwargs),
+                    nn.Linear(dim, dim_inner * 2, bias=False, **factory_kwargs),
+                    FusedSwiGLU(),
+                    nn.Linear(dim_inner, dim, bias=False, **factory_kwargs),
+                )
+        else:
+            self.ff = nn.Sequential(
+                nn.Linear(dim, dim_inner * 2, bias=False, **factory_kwargs),
+                FusedSwiGLU(),
+                nn.Linear(dim_inner, dim, bias=False, **factory_kwargs),
+            )
+
+    def forward(self, input):
+        if self._fused_ln_swiglu:
+            # LayerNorm -> Linear -> SwiGLU in one kernel, then the output projection
+            return self.ff[2](self.ff[0](input, act=_lib.MF_ACT_SWIGLU))
+        return self.ff(input)
+
+    def extra_repr(self):
+        return f"dim={self.dim}, dim_inner={self.dim_inner}"
