@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X attention path on the headline workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward + one backward of the pair-biased, key-masked attention on configuration C2:
+q, k, v [1, 384, 384, 4, 32] bf16, fp32 pair bias [1, 1, 4, 384, 384], last 38 of 384 keys padded,
+seeded synthetic inputs resident in HBM before the timed region.  Prints ONE JSON line.
+
+* ``value`` — algorithmic TFLOP/s of fwd+bwd, FLOP convention of the reference
+  (benchmarks/evoattention_speed.py:110-115): one matmul = 2*B*N*H*S*S*D, forward 2, backward 5
+  (recomputation not counted) => 7 * 14.496 = 101.469 GFLOP per step.
+* ``roofline`` — for the kernel that takes the most time: algorithmic FLOPs of that launch divided by
+  its average duration, measured with events on the launch stream inside the timed region.
+* ``cpu_baseline`` — the CPU oracle (eager PyTorch restatement, fp32) timed on the host cores on a
+  bounded sample of the same workload.  Reported next to the GPU number; not a target.
+* extra keys: peak activation MiB (caching allocator), per-phase ms, and fwd / bwd times of the
+  LayerNorm->Linear (C3) and Transition (C4) workloads with their HBM GB/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the C3/C4/C5 side measurements")
+    return ap.parse_args()
+
+
+def attention_flops(B, N, S, H, D):
+    mm = 2.0 * B * N * H * S * S * D
+    return {"matmul": mm, "fwd": 2 * mm, "bwd": 5 * mm, "total": 7 * mm}
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def cpu_baseline(inp, flops_total, budget_s=20.0):
+    """Times the CPU oracle (fp32, all host threads up to 16) on a slice of the rows of C2: rows are
+    independent problems, so FLOPs scale linearly with the slice."""
+    import torch
+    from oracle import evoattention as oe
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    N = inp["q"].shape[1]
+    rows = 16
+
+    def once(r):
+        sl = slice(0, r)
+        t0 = time.perf_counter()
+        oe.evo_attention_chunked(inp["q"][:, sl], inp["k"][:, sl], inp["v"][:, sl], inp["mask"][:, sl], inp["bias"],
+                                 inp["dO"][:, sl], chunk=16, dtype=torch.float32)
+        return time.perf_counter() - t0
+
+    t = once(rows)                     # warm-up, also sizes the sample
+    while rows < N and t * 2 * 3 < budget_s:
+        rows *= 2
+        t = once(rows)
+    rows = min(rows, N)
+    times = [once(rows) for _ in range(3)]
+    tmed = median(times)
+    tflops = flops_total * rows / N / tmed / 1e12
+    return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "fwd+bwd of rows 0..%d of %d of the same C2 tensors (rows are independent; dBias summed over "
+                      "the sample), fp32 eager PyTorch oracle, median of 3 (%.2f s each)" % (rows - 1, N, tmed)}
+
+
+def load_traffic():
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f)
+    return {}
+
+
+def time_fn(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return median([a.elapsed_time(b) for a, b in evs])
+
+
+def side_measurements(torch, steps, warmup):
+    """fwd / bwd ms of C3 (LayerNorm->Linear), C4 (Transition), and C5 peak memory."""
+    from megafold_amd import workloads
+    from megafold_amd.model.FusedLayernormLinear.fused_layernorm_linear import (layernorm_linear_backward,
+                                                                                 layernorm_linear_forward)
+    from megafold_amd.model.FusedEvoAttention.evoattention import TritonEvoformer
+    from megafold_amd import _lib
+    out = {}
+    inp = {k: (v.cuda() if v is not None else None) for k, v in workloads.lnlinear_inputs().items()}
+    M, K, N = 147456, 128, 512
+    fwd = lambda: layernorm_linear_forward(inp["x"], inp["W"], inp["b"], inp["gamma"], inp["beta"], True, True)
+    c, x2, W, Mean, RSTD = fwd()
+    bwd = lambda: layernorm_linear_backward(inp["dY"], x2, W, Mean, RSTD, inp["gamma"], inp["beta"], True, True)
+    tf, tb = time_fn(fwd, steps, warmup, torch), time_fn(bwd, steps, warmup, torch)
+    bf = (M * K + K * N + M * N) * 2
+    bb = (M * N + M * K + K * N + M * K + K * N) * 2
+    out["lnlinear_c3"] = {"fwd_ms": round(tf, 4), "bwd_ms": round(tb, 4), "fwd_GBps": round(bf / tf / 1e6, 1),
+                          "bwd_GBps": round(bb / tb / 1e6, 1), "fwd_frac_hbm": round(bf / tf / 1e6 / PEAK_HBM_GBS, 4),
+                          "bwd_frac_hbm": round(bb / tb / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_MB": [bf / 1e6, bb / 1e6]}
+    del c, x2, Mean, RSTD
+    tin = {k: v.cuda() for k, v in workloads.transition_inputs().items()}
+    N1 = 1024
+    fwd = lambda: layernorm_linear_forward(tin["x"], tin["W1"], None, tin["gamma"], tin["beta"], True, False,
+                                           act=_lib.MF_ACT_SWIGLU)
+    h, x2, W1, Mean, RSTD = fwd()
+    dh = torch.randn_like(h)
+    bwd = lambda: layernorm_linear_backward(dh, x2, W1, Mean, RSTD, tin["gamma"], tin["beta"], True, False,
+                                            act=_lib.MF_ACT_SWIGLU)
+    tf, tb = time_fn(fwd, steps, warmup, torch), time_fn(bwd, steps, warmup, torch)
+    bf = (M * K + K * N1 + M * 512) * 2
+    bb = (M * 512 + M * K + K * N1 + M * K + K * N1) * 2
+    out["ln_swiglu_c4"] = {"fwd_ms": round(tf, 4), "bwd_ms": round(tb, 4), "fwd_GBps": round(bf / tf / 1e6, 1),
+                           "bwd_GBps": round(bb / tb / 1e6, 1), "fwd_frac_hbm": round(bf / tf / 1e6 / PEAK_HBM_GBS, 4),
+                           "bwd_frac_hbm": round(bb / tb / 1e6 / PEAK_HBM_GBS, 4),
+                           "fwd_TFLOPs": round(2.0 * M * K * N1 / tf / 1e9, 1)}
+    del h, x2, Mean, RSTD, dh, tin, inp
+    torch.cuda.empty_cache()
+    c5 = {k: v.cuda() for k, v in workloads.config5().items()}
+    q, k, v = (c5[n].requires_grad_() for n in "qkv")
+    bias = c5["bias"].requires_grad_()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    o = TritonEvoformer(q, k, v, c5["mask"], bias)
+    o.backward(c5["dO"])
+    torch.cuda.synchronize()
+    out["c5_peak_act_mib"] = round((torch.cuda.max_memory_allocated() - base) / 2 ** 20, 1)
+    out["c5_bound_mib"] = 4 * 144 + 3 * 9
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the op shards trivially over "
+              "rows; see DESIGN.md).  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from megafold_amd import workloads
+    from megafold_amd.model.FusedEvoAttention.evoattention import (TritonEvoformer, evoattention_backward,
+                                                                    evoattention_forward)
+    torch.cuda.set_device(0)
+    B, N, S, H, D = 1, 384, 384, 4, 32
+    fl = attention_flops(B, N, S, H, D)
+    inp = workloads.config2()
+    dev = {k: v.cuda() for k, v in inp.items()}
+
+    # ---- peak activation memory of one fwd+bwd through the autograd operator --------------------
+    q, k, v = (dev[n].clone().requires_grad_() for n in "qkv")
+    bias = dev["bias"].clone().requires_grad_()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    out = TritonEvoformer(q, k, v, dev["mask"], bias)
+    out.backward(dev["dO"])
+    torch.cuda.synchronize()
+    peak_mib = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+    del out, q, k, v, bias
+
+    # ---- timed region: K steps of fwd + bwd, every phase bracketed by events on the launch stream ----
+    names = ("fwd", "dqkv", "dbias")
+    marks = []
+
+    def step(record):
+        ev = {}
+        if record:
+            ev["fwd"] = [torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)]
+            ev["fwd"][0].record()
+        O, lse, (Q, K_, V, mask, bias_) = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"])
+        if record:
+            ev["fwd"][1].record()
+
+        def hook(name):
+            if not record:
+                return
+            e = torch.cuda.Event(enable_timing=True)
+            e.record()
+            ev.setdefault(name, []).append(e)
+
+        evoattention_backward(dev["dO"], Q, K_, V, mask, bias_, O, lse, True, phase_hook=hook)
+        if record:
+            marks.append(ev)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    per = {n: sum(m[n][0].elapsed_time(m[n][1]) for m in marks) / len(marks) for n in names}
+    span = sum(m["fwd"][0].elapsed_time(m["dbias"][1]) for m in marks) / len(marks)
+    ms_per_step = max(wall_ms, span)     # never better than the host-side clock around the region
+    value = fl["total"] / ms_per_step / 1e9
+
+    # ---- roofline of the kernel that takes the most time -------------------------------------------
+    # algorithmic FLOPs per launch: fwd 2 matmuls; dqkv all 5 backward matmuls; dbias recomputes
+    # (S, dP) to reduce dS over N and is credited none of the algorithmic FLOPs
+    alg = {"fwd": fl["fwd"], "dqkv": fl["bwd"], "dbias": 0.0}
+    kern = {"fwd": "evo_fwd_kernel", "dqkv": "evo_bwd_dqkv_kernel", "dbias": "evo_bwd_dbias_kernel"}
+    dom = max(names, key=lambda n: per[n])
+    if alg[dom] == 0.0:
+        dom = max(("fwd", "dqkv"), key=lambda n: per[n])
+    achieved = alg[dom] / per[dom] / 1e9
+    traffic = load_traffic().get(kern[dom])
+    roofline = {"bound": "mfma", "kernel": kern[dom], "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                "avg_launch_ms": round(per[dom], 5), "algorithmic_GFLOP": round(alg[dom] / 1e9, 3)}
+
+    res = {
+        "metric": "EvoAttention fwd+bwd TFLOP/s + peak act MiB, N=S=384 H=4 D=32 bf16",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C2 triangle attention fwd+bwd: q,k,v [1,384,384,4,32] bf16, fp32 pair bias "
+                               "[1,1,4,384,384], last 38 keys masked (-inf), dO ~ N(0,1)",
+                   "B": B, "N": N, "S": S, "H": H, "D": D, "algorithmic_GFLOP_per_step": round(fl["total"] / 1e9, 3)},
+        "roofline": roofline,
+        "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+        "peak_act_mib": round(peak_mib, 2), "peak_act_bound_mib": 150.75,
+        "phase_ms": {n: round(per[n], 5) for n in names},
+        "hbm_GBps_at_algorithmic_bytes": round(468.0 / ms_per_step, 1),
+    }
+    if not args.no_extras:
+        res.update(side_measurements(torch, max(5, args.steps // 5), 3))
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(inp, fl["total"])
+    else:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -14,7 +14,8 @@
  *   mf_lnlinear_fwd       layernorm_linear_forward     megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:351-405
  *   mf_lnlinear_bwd       layernorm_linear_backward    megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:408-474
  *   mf_swiglu_fwd / _bwd  swiglu_forward / _backward   megafold/model/FusedTransition/fused_transition.py:55-93
- *   mf_ln_swiglu_fwd/_bwd LayernormLinear + FusedSwiGLU of FusedTransition.ff[0:2]
+ *   mf_lnlinear_* with act = MF_ACT_SWIGLU
+ *                         LayernormLinear + FusedSwiGLU of FusedTransition.ff[0:2]
  *                                                      megafold/model/FusedTransition/fused_transition.py:128-131
  */
 #ifndef MEGAFOLD_AMD_H
@@ -59,11 +60,17 @@ const char* mf_last_error(void);
  * 16 bytes; pointers 16-byte aligned.
  * A query row whose keys are all masked with -inf yields o = 0, lse = -inf and zero gradients.
  * ---------------------------------------------------------------------------------------------- */
+/* Backward phases.  MF_EVO_BWD_DQKV writes dq, dk, dv and leaves rowsum(dO * o) in the workspace;
+ * MF_EVO_BWD_DBIAS reads it and writes dbias, so it must follow a DQKV call on the same stream with
+ * the same workspace.  phases = 0 runs both (the second only when dbias != NULL). */
+#define MF_EVO_BWD_DQKV 1
+#define MF_EVO_BWD_DBIAS 2
+
 typedef struct mf_evoattn_args {
   int32_t B, N, S, H, D;
   int32_t dtype, bias_dtype, mask_dtype;
   float scale; /* softmax scale; the reference uses D^-0.5 */
-  int32_t reserved0;
+  int32_t phases; /* backward only: 0 = everything; else a mask of MF_EVO_BWD_* (see below) */
   const void *q, *k, *v;
   const void* bias;
   const void* mask;

@@ -14,6 +14,7 @@ LIB_PATH = PKG / "lib" / "libmegafold_amd.so"
 
 MF_F32, MF_F16, MF_BF16, MF_BOOL = 0, 1, 2, 3
 MF_ACT_NONE, MF_ACT_SWIGLU = 0, 1
+MF_EVO_BWD_DQKV, MF_EVO_BWD_DBIAS = 1, 2
 
 I64x4 = C.c_int64 * 4
 I64x3 = C.c_int64 * 3
@@ -23,7 +24,7 @@ class EvoAttnArgs(C.Structure):
     _fields_ = [
         ("B", C.c_int32), ("N", C.c_int32), ("S", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32), ("bias_dtype", C.c_int32), ("mask_dtype", C.c_int32),
-        ("scale", C.c_float), ("reserved0", C.c_int32),
+        ("scale", C.c_float), ("phases", C.c_int32),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
         ("bias", C.c_void_p), ("mask", C.c_void_p),
         ("o", C.c_void_p), ("lse", C.c_void_p),

@@ -150,6 +150,7 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   if ((rc = check_tensor("dk", a->dk, a->dk_stride, es))) return rc;
   if ((rc = check_tensor("dv", a->dv, a->dv_stride, es))) return rc;
   if (a->dbias && !aligned16(a->dbias)) return fail(MF_ERR_ALIGN, "dbias is not 16-byte aligned");
+  if (a->phases < 0 || a->phases > (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS)) return fail(MF_ERR_SHAPE, "phases %d unknown", a->phases);
   const Plan pl = make_plan(a, true);
   if (!a->workspace || a->workspace_bytes < pl.total)
     return fail(MF_ERR_WORKSPACE, "backward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
@@ -167,8 +168,12 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   p.n_chunks = pl.n_chunks;
   p.rows_per_chunk = pl.rows_per_chunk;
   p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
-  hipError_t e = launch_evo_bwd_dqkv(p, stream);
-  if (e != hipSuccess) return (int)e;
-  if (a->dbias) e = launch_evo_bwd_dbias(p, stream);
+  const int phases = a->phases == 0 ? (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;
+  hipError_t e = hipSuccess;
+  if (phases & MF_EVO_BWD_DQKV) {
+    e = launch_evo_bwd_dqkv(p, stream);
+    if (e != hipSuccess) return (int)e;
+  }
+  if ((phases & MF_EVO_BWD_DBIAS) && a->dbias) e = launch_evo_bwd_dbias(p, stream);
   return (int)e;
 }

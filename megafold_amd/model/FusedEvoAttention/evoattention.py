@@ -117,8 +117,12 @@ def evoattention_forward(Q, K, V, res_mask, pair_bias):
     return O, lse, (Q, K, V, mask, bias)
 
 
-def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True):
-    """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state."""
+def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None):
+    """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state.
+
+    ``phase_hook(name)``, if given, is called before and after each of the two backward phases
+    ("dqkv", "dbias"), which are then enqueued by two separate C-ABI calls (used by the benchmark to
+    bracket each kernel with events on the launch stream)."""
     B, N, S, H, D = Q.shape
     if dO.dtype != Q.dtype:
         dO = dO.to(Q.dtype)
@@ -141,7 +145,16 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True):
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=Q.device)
         a.workspace = ws.data_ptr()
         a.workspace_bytes = nbytes
-        _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd")
+        if phase_hook is None:
+            _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd")
+        else:
+            for name, bit in (("dqkv", _lib.MF_EVO_BWD_DQKV), ("dbias", _lib.MF_EVO_BWD_DBIAS)):
+                if bit == _lib.MF_EVO_BWD_DBIAS and dbias is None:
+                    continue
+                a.phases = bit
+                phase_hook(name)
+                _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd[%s]" % name)
+                phase_hook(name)
     return dQ, dK, dV, dbias
 
 

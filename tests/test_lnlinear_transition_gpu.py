@@ -1,0 +1,207 @@
+"""Parity of the HIP LayerNorm->Linear / SwiGLU / Transition path against the CPU oracle (GPU box
+only); every call goes through the C ABI (``mf_lnlinear_*`` / ``mf_swiglu_*``) via the drop-in modules."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from conftest import tol_for
+from megafold_amd import workloads
+from megafold_amd.model.FusedLayernormLinear.fused_layernorm_linear import LayernormLinear
+from megafold_amd.model.FusedTransition.fused_transition import FusedSwiGLU, FusedTransition
+from oracle import layernorm_linear as ol
+from oracle import transition as ot
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+f64 = torch.float64
+
+
+def close(got, want, dtype, name, scale_atol=1.0):
+    t = dict(tol_for(dtype))
+    t["atol"] = t["atol"] * scale_atol
+    assert not torch.isnan(got).any(), name
+    torch.testing.assert_close(got.detach().cpu().to(want.dtype), want, msg=lambda m: "%s: %s" % (name, m), **t)
+
+
+def make_module(inp, K, N, dtype, bias):
+    mod = LayernormLinear(K, N, has_linear_bias=bias, device="cuda", dtype=dtype)
+    with torch.no_grad():
+        mod.WEIGHT.copy_(inp["gamma"]); mod.BIAS.copy_(inp["beta"]); mod.linear_weight.copy_(inp["W"])
+        if bias:
+            mod.linear_bias.copy_(inp["b"])
+    return mod
+
+
+# (M-shape, K, N) from the reference's sweep (tests/test_layernormlinear.py:44-60) and the model's (N, K) table
+SWEEP = [
+    ((16,), 16, 16, torch.float32, True),
+    ((3, 37), 64, 48, torch.float32, True),
+    ((8000,), 128, 512, torch.bfloat16, True),
+    ((777,), 128, 16, torch.bfloat16, True),      # pair-bias heads (16, 128)
+    ((2, 300), 64, 64, torch.bfloat16, False),    # outer-product-mean (64, 64)
+    ((513,), 16, 8, torch.float16, True),
+    ((300,), 256, 264, torch.bfloat16, True),
+    ((5000,), 128, 640, torch.bfloat16, False),   # triangle multiplication (640, 128)
+    ((1000,), 64, 320, torch.bfloat16, False),    # (320, 64)
+    ((1200,), 128, 128, torch.bfloat16, False),   # (128, 128)
+    ((900,), 128, 8, torch.bfloat16, False),      # (8, 128)
+    ((100,), 768, 768, torch.float32, True),      # K beyond the kernels: same eager expression as the reference's fallback
+]
+
+
+@pytest.mark.parametrize("mshape,K,N,dtype,bias", SWEEP)
+def test_layernorm_linear_parity(mshape, K, N, dtype, bias):
+    print("case", mshape, K, N, dtype, bias, flush=True)
+    inp = workloads.lnlinear_inputs(mshape, K, N, dtype=dtype, seed=K + N, linear_bias=bias)
+    if bias:
+        inp["b"] = (0.3 * torch.randn(N, generator=torch.Generator().manual_seed(1))).to(dtype)
+    mod = make_module({k: (v.cuda() if v is not None else None) for k, v in inp.items()}, K, N, dtype, bias)
+    x = inp["x"].cuda().requires_grad_()
+    out = mod(x)
+    out.backward(inp["dY"].cuda())
+    ref = ol.layernorm_linear_forward(inp["x"], inp["gamma"], inp["beta"], inp["W"], inp["b"], dtype=f64)
+    rdx, rdW, rdb, rdg, rdbt = ol.layernorm_linear_backward(inp["dY"], inp["x"], inp["gamma"], inp["beta"], inp["W"], dtype=f64)
+    M = int(np.prod(mshape))
+    close(out, ref, dtype, "out")
+    close(x.grad, rdx, dtype, "dX")
+    # parameter gradients are sums over M rows: the absolute bar scales with the magnitude of the sum
+    s = max(1.0, M ** 0.5)
+    close(mod.linear_weight.grad, rdW, dtype, "dW", s)
+    close(mod.WEIGHT.grad, rdg, dtype, "dgamma", s)
+    close(mod.BIAS.grad, rdbt, dtype, "dbeta", s)
+    if bias:
+        close(mod.linear_bias.grad, rdb, dtype, "dLinearBias", s)
+    assert out.dtype == dtype and out.shape == tuple(mshape) + (N,)
+
+
+def test_small_fp32_against_golden():
+    g = np.load(os.path.join(GOLD, "lnlinear_small.npz"))
+    inp = workloads.lnlinear_inputs((3, 37), 64, 48, dtype=torch.float32, seed=5)
+    inp["b"] = torch.from_numpy(g["b"]).float()
+    mod = make_module({k: v.cuda() for k, v in inp.items()}, 64, 48, torch.float32, True)
+    x = inp["x"].cuda().requires_grad_()
+    out = mod(x)
+    out.backward(inp["dY"].cuda())
+    for name, t in (("out", out), ("dx", x.grad), ("dW", mod.linear_weight.grad), ("db", mod.linear_bias.grad),
+                    ("dgamma", mod.WEIGHT.grad), ("dbeta", mod.BIAS.grad)):
+        np.testing.assert_allclose(t.detach().cpu().numpy(), g[name], rtol=1e-4, atol=2e-5, err_msg=name)
+
+
+def test_config3_full_size_parity_and_properties():
+    """C3: x [1, 384, 384, 128] bf16 -> 512, the fused q/k/v/gate projection."""
+    inp = workloads.lnlinear_inputs()
+    mod = make_module({k: v.cuda() for k, v in inp.items()}, 128, 512, torch.bfloat16, True)
+    x = inp["x"].cuda().requires_grad_()
+    out = mod(x)
+    out.backward(inp["dY"].cuda())
+    ref = ol.layernorm_linear_forward(inp["x"], inp["gamma"], inp["beta"], inp["W"], inp["b"])
+    rdx, rdW, rdb, rdg, rdbt = ol.layernorm_linear_backward(inp["dY"], inp["x"], inp["gamma"], inp["beta"], inp["W"])
+    close(out, ref, torch.bfloat16, "out")
+    close(x.grad, rdx, torch.bfloat16, "dX")
+    s = 147456 ** 0.5
+    close(mod.linear_weight.grad, rdW, torch.bfloat16, "dW", s)
+    close(mod.WEIGHT.grad, rdg, torch.bfloat16, "dgamma", s)
+    close(mod.BIAS.grad, rdbt, torch.bfloat16, "dbeta", s)
+    close(mod.linear_bias.grad, rdb, torch.bfloat16, "db", s)
+    # LayerNorm backward projects out the constant direction of every row
+    assert x.grad.float().sum(-1).abs().max() < 0.25
+    # bitwise reproducible (no atomics)
+    x2 = inp["x"].cuda().requires_grad_()
+    mod.zero_grad()
+    out2 = mod(x2)
+    g1 = mod.linear_weight.grad
+    out2.backward(inp["dY"].cuda())
+    assert torch.equal(out, out2) and torch.equal(x.grad, x2.grad)
+    # linearity in dOut: backward(2 dY) == 2 backward(dY) exactly (power-of-two scaling)
+    x3 = inp["x"].cuda().requires_grad_()
+    mod(x3).backward(2 * inp["dY"].cuda())
+    assert torch.equal(x3.grad, 2 * x.grad)
+
+
+def test_autocast_contract_and_state_dict_names():
+    mod = LayernormLinear(128, 64, device="cuda")            # fp32 parameters
+    assert sorted(mod.state_dict()) == ["BIAS", "WEIGHT", "linear_bias", "linear_weight"]
+    assert mod.linear_weight.shape == (128, 64)
+    x = torch.randn(50, 128, device="cuda", requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = mod(x)
+    assert out.dtype == torch.bfloat16                       # custom_fwd(cast_inputs=bfloat16)
+    out.float().sum().backward()
+    assert x.grad.dtype == torch.float32 and mod.linear_weight.grad.dtype == torch.float32
+    ref = ol.layernorm_linear_forward(x.detach().cpu(), mod.WEIGHT.detach().cpu(), mod.BIAS.detach().cpu(),
+                                      mod.linear_weight.detach().cpu(), mod.linear_bias.detach().cpu())
+    close(out, ref, torch.bfloat16, "autocast out")
+
+
+@pytest.mark.parametrize("mshape,dim,ef,dtype", [((2, 29), 32, 4, torch.float32), ((1000,), 128, 4, torch.bfloat16),
+                                                   ((4097,), 64, 4, torch.bfloat16), ((300,), 128, 2, torch.float16)])
+def test_fused_transition_parity(mshape, dim, ef, dtype):
+    inp = workloads.transition_inputs(mshape, dim, ef, dtype=dtype, seed=7)
+    mod = FusedTransition(dim, ef, device="cuda", dtype=dtype)
+    assert sorted(mod.state_dict()) == ["ff.0.BIAS", "ff.0.WEIGHT", "ff.0.linear_weight", "ff.2.weight"]
+    with torch.no_grad():
+        mod.ff[0].WEIGHT.copy_(inp["gamma"]); mod.ff[0].BIAS.copy_(inp["beta"])
+        mod.ff[0].linear_weight.copy_(inp["W1"]); mod.ff[2].weight.copy_(inp["W2"])
+    x = inp["x"].cuda().requires_grad_()
+    y = mod(x)
+    y.backward(inp["dY"].cuda())
+    # oracle: autograd of the float64 eager Transition (benchmarks/transition_speed.py:8-39)
+    xr, gr, br, w1, w2 = (inp[n].double().requires_grad_() for n in ("x", "gamma", "beta", "W1", "W2"))
+    yr = ot.transition_forward(xr, gr, br, w1, w2, dtype=f64)
+    yr.backward(inp["dY"].double())
+    M = int(np.prod(mshape))
+    s = max(1.0, M ** 0.5)
+    close(y, yr.detach(), dtype, "y")
+    close(x.grad, xr.grad, dtype, "dX")
+    close(mod.ff[0].linear_weight.grad, w1.grad, dtype, "dW1", s)
+    close(mod.ff[2].weight.grad, w2.grad, dtype, "dW2", s)
+    close(mod.ff[0].WEIGHT.grad, gr.grad, dtype, "dgamma", s)
+    close(mod.ff[0].BIAS.grad, br.grad, dtype, "dbeta", s)
+    if dtype == torch.float32:
+        g = np.load(os.path.join(GOLD, "transition_small.npz"))
+        np.testing.assert_allclose(y.detach().cpu().numpy(), g["y"], rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("include_ln,use_lnl", [(True, False), (False, True)])
+def test_transition_variants_use_standalone_swiglu(include_ln, use_lnl):
+    dim = 64
+    mod = FusedTransition(dim, 2, include_ln=include_ln, use_layernormlinear=use_lnl, device="cuda", dtype=torch.bfloat16)
+    x = torch.randn(333, dim, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    y = mod(x)
+    y.float().sum().backward()
+    ref = nn.Sequential(*[m if not isinstance(m, FusedSwiGLU) else _EagerSwiGLU() for m in mod.ff]).float()
+    xr = x.detach().float().requires_grad_()
+    yr = ref(xr)
+    yr.sum().backward()
+    close(y, yr.detach().cpu(), torch.bfloat16, "y")
+    close(x.grad, xr.grad.cpu(), torch.bfloat16, "dX")
+
+
+class _EagerSwiGLU(nn.Module):
+    def forward(self, x):
+        a, g = x.chunk(2, dim=-1)
+        return torch.nn.functional.silu(g) * a
+
+
+def test_config4_full_size_transition():
+    """C4: x [1, 384, 384, 128] bf16, 128 -> 1024 -> SwiGLU -> 512 -> 128."""
+    inp = workloads.transition_inputs()
+    mod = FusedTransition(128, 4, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        mod.ff[0].WEIGHT.copy_(inp["gamma"]); mod.ff[0].BIAS.copy_(inp["beta"])
+        mod.ff[0].linear_weight.copy_(inp["W1"]); mod.ff[2].weight.copy_(inp["W2"])
+    x = inp["x"].cuda().requires_grad_()
+    y = mod(x)
+    y.backward(inp["dY"].cuda())
+    # fp32 oracle on a slice of rows (rows are independent); parameter gradients by linearity are
+    # checked on the small cases above
+    sl = slice(200, 204)
+    xr = inp["x"][:, sl].float().requires_grad_()
+    yr = ot.transition_forward(xr, inp["gamma"], inp["beta"], inp["W1"], inp["W2"])
+    yr.backward(inp["dY"][:, sl].float())
+    close(y[:, sl], yr.detach(), torch.bfloat16, "y")
+    close(x.grad[:, sl], xr.grad, torch.bfloat16, "dX")
+    assert not torch.isnan(mod.ff[0].linear_weight.grad).any()
