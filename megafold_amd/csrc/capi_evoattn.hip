@@ -3,6 +3,7 @@
 // Host side of the reference being replaced: EvoformerAttention.forward / .backward
 // (megafold/model/FusedEvoAttention/evoattention.py:688-779, 782-903).
 #include "../../include/megafold_amd.h"
+#include <cstdlib>
 #include "capi_common.h"
 #include "common.h"
 #include "evoattn.h"
@@ -12,24 +13,18 @@ using namespace mf;
 namespace {
 
 struct Plan {
-  bool bias_copy;     // bias must be converted / padded into the workspace
-  int bias_ld;        // row length of the fp32 bias the kernels read
+  int bias_rows, bias_ld;   // padded shape of the fp32 bias/scale copy the kernels read
   uint64_t off_bias, off_delta, off_part, total;
   int n_chunks, rows_per_chunk;
 };
 
-bool bias_direct(const mf_evoattn_args* a) {
-  return a->bias_dtype == MF_DTYPE_F32 && a->bias_stride[3] == 1 && a->bias_stride[2] % 4 == 0 &&
-         a->bias_stride[1] % 4 == 0 && a->bias_stride[0] % 4 == 0 && a->S % 16 == 0 && aligned16(a->bias);
-}
-
 Plan make_plan(const mf_evoattn_args* a, bool backward) {
   Plan pl{};
-  pl.bias_copy = !bias_direct(a);
-  pl.bias_ld = pl.bias_copy ? round_up(a->S, 16) : (int)a->bias_stride[2];
+  pl.bias_rows = round_up(a->S, 32);
+  pl.bias_ld = round_up(a->S, 64);
   uint64_t off = 0;
   pl.off_bias = off;
-  if (pl.bias_copy) off += align256((uint64_t)a->B * a->H * a->S * pl.bias_ld * 4);
+  off += align256((uint64_t)a->B * a->H * pl.bias_rows * pl.bias_ld * 4);
   pl.n_chunks = 1;
   pl.rows_per_chunk = a->N;
   if (backward) {
@@ -90,25 +85,23 @@ int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStrea
   p.B = a->B; p.N = a->N; p.S = a->S; p.H = a->H; p.D = a->D;
   p.dtype = a->dtype;
   p.scale = a->scale;
+  { const char* e = getenv("MF_DBG"); p.dbg = e ? atoi(e) : 0; }
   p.q = tens(a->q, a->q_stride); p.k = tens(a->k, a->k_stride); p.v = tens(a->v, a->v_stride);
   p.o = tens(a->o, a->o_stride);
   p.mask = a->mask; p.mask_dtype = a->mask_dtype;
   p.mask_sb = a->mask_stride[0]; p.mask_sn = a->mask_stride[1]; p.mask_sj = a->mask_stride[2];
   p.lse = a->lse;
   unsigned char* ws = static_cast<unsigned char*>(a->workspace);
-  if (pl.bias_copy) {
-    float* b32 = reinterpret_cast<float*>(ws + pl.off_bias);
-    hipError_t e = launch_bias_to_f32(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
-                                      a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_ld, stream);
-    if (e != hipSuccess) return (int)e;
-    p.bias = b32;
-    p.bias_sb = (int64_t)a->H * a->S * pl.bias_ld;
-    p.bias_sh = (int64_t)a->S * pl.bias_ld;
-    p.bias_ld = pl.bias_ld;
-  } else {
-    p.bias = static_cast<const float*>(a->bias);
-    p.bias_sb = a->bias_stride[0]; p.bias_sh = a->bias_stride[1]; p.bias_ld = a->bias_stride[2];
-  }
+  float* b32 = reinterpret_cast<float*>(ws + pl.off_bias);
+  if (a->scale <= 0.0f) return fail(MF_ERR_SHAPE, "scale must be positive (got %g)", (double)a->scale);
+  hipError_t e = launch_bias_prep(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
+                                  a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_rows, pl.bias_ld, 1.0f / a->scale,
+                                  stream);
+  if (e != hipSuccess) return (int)e;
+  p.bias = b32;
+  p.bias_sb = (int64_t)a->H * pl.bias_rows * pl.bias_ld;
+  p.bias_sh = (int64_t)pl.bias_rows * pl.bias_ld;
+  p.bias_ld = pl.bias_ld;
   return 0;
 }
 
@@ -130,10 +123,10 @@ extern "C" int mf_evoattn_fwd(const mf_evoattn_args* a) {
   int rc = check_common(a);
   if (rc) return rc;
   const Plan pl = make_plan(a, false);
-  if (pl.total > 0 && (!a->workspace || a->workspace_bytes < pl.total))
+  if (!a->workspace || a->workspace_bytes < pl.total)
     return fail(MF_ERR_WORKSPACE, "forward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
                 (unsigned long long)(a->workspace ? a->workspace_bytes : 0));
-  if (pl.total > 0 && !aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
+  if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   EvoParams p;
   rc = fill_params(a, pl, p, stream);

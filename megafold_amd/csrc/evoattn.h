@@ -19,10 +19,10 @@ struct EvoParams {
   int dtype;       // MF_F32 / MF_F16 / MF_BF16: element type of q, k, v, o, dO, dq, dk, dv
   float scale;     // softmax scale, D^-0.5 in the reference (evoattention.py:705)
   EvoTensor q, k, v, o;
-  // Pair bias as fp32 [B, H, S, bias_ld]: row (b, h, i) starts at bias + b*bias_sb + h*bias_sh + i*bias_ld.
-  // bias_ld is a multiple of 4 and every row has at least round_up(S, 16) readable floats when
-  // S is not a multiple of 16 (the host copies/pads into the workspace when the caller's tensor does
-  // not satisfy this).
+  // Pair bias DIVIDED BY scale as fp32 [B, H, Sr, bias_ld] with Sr = round_up(S, 32) rows and
+  // bias_ld = round_up(S, 64) columns, zero padded (built in the workspace by launch_bias_prep), so
+  // the kernels read it without bounds checks; row (b, h, i) starts at
+  // bias + b*bias_sb + h*bias_sh + i*bias_ld.
   const float* bias;
   int64_t bias_sb, bias_sh, bias_ld;
   // Additive key mask [B, N, S] in its own dtype (MF_BOOL: keep-mask, true -> 0, false -> -inf).
@@ -35,6 +35,7 @@ struct EvoParams {
   float* delta;    // [B, N, H, S] fp32 rowsum(dO * O)
   float* dbias;    // [B, H, S, S] fp32 or nullptr
   float* dbias_part;  // [n_chunks, B, H, S, S] fp32 partial sums (nullptr when n_chunks == 1)
+  int dbg;         // experiment switches (0 in production)
   int n_chunks;    // number of N-chunks the bias-gradient kernel splits the rows into
   int rows_per_chunk;
 };
@@ -43,9 +44,9 @@ struct EvoParams {
 hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dbias(const EvoParams& p, hipStream_t stream);
-// bias (any float dtype, any strides) -> fp32 [B, H, S, ld] with zero padding for j >= S.
-hipError_t launch_bias_to_f32(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
-                              int B, int H, int S, int ld, hipStream_t stream);
+// bias (any float dtype, any strides) * mult -> fp32 [B, H, Sr, ld], zero padded for i >= S or j >= S.
+hipError_t launch_bias_prep(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
+                            int B, int H, int S, int Sr, int ld, float mult, hipStream_t stream);
 
 // Number of rows of N one work-group of the bias-gradient kernel walks over, chosen so the grid
 // fills the device while the partial-sum workspace stays small.

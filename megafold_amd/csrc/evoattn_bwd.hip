@@ -84,7 +84,10 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   frag qaugA = frag_zero<T>();   // Q side of the mask-carrier step (A operand here)
   if (g == 0) { qaugA[0] = (T)1.0f; qaugA[1] = (T)1.0f; }
 
-  // ---- staging of one query tile: Q (pre-scaled), dO, LSE, delta -------------------------------
+  const float cexp = p.scale * MF_LOG2E;   // the accumulator holds z / scale (unscaled q.k + bias/scale + mask/scale)
+  const float inv_scale = 1.0f / p.scale;
+
+  // ---- staging of one query tile: Q, dO, LSE, delta --------------------------------------------
   frag sq[PF], sdo[PF];
   float sdelta[PF], slse[PF];
   auto fetch_q = [&](int it) {
@@ -99,7 +102,7 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
         const bool ok = qi < S && 8 * dc < D;
         frag of = frag_zero<T>();
         if (ok) {
-          sq[i] = scale8<T>(ld8<T>(Qg + (int64_t)qi * p.q.ss + 8 * dc), p.scale);
+          sq[i] = ld8<T>(Qg + (int64_t)qi * p.q.ss + 8 * dc);
           sdo[i] = ld8<T>(dOg + (int64_t)qi * p.dO.ss + 8 * dc);
           of = ld8<T>(Og + (int64_t)qi * p.o.ss + 8 * dc);
         }
@@ -149,7 +152,8 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
     }
     for (int kk = tid; kk < KC; kk += nthr) {
       const int j = tile0 * 32 + kk;
-      const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) : -__builtin_inff();
+      const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) * inv_scale
+                             : -__builtin_inff();
       frag a = frag_zero<T>();
       T hi, lo;
       split_hi_lo<T>(mv, hi, lo);
@@ -173,6 +177,25 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) { dk[t][dt] = acc_zero(); dv[t][dt] = acc_zero(); }
+
+    // bias/scale tile of the next (query tile, key tile) step, loaded one step ahead.  The copy in
+    // the workspace is zero padded to whole tiles, so no bounds checks: register i of half g <->
+    // query 32*it + 16*g + i, lane x <-> key j0 + x.
+    const float* bias_t[TPW];
+    bool tile_ok[TPW];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      const int j0 = (tile0 + w * TPW + t) * 32;
+      tile_ok[t] = j0 < S;
+      bias_t[t] = biasg + (int64_t)(16 * g) * p.bias_ld + (tile_ok[t] ? j0 : 0) + x;
+    }
+    f32x16 bzn;
+    auto load_bias = [&](int it, const float* base) {
+      const float* bp = base + (int64_t)it * 32 * p.bias_ld;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bzn[i] = bp[(int64_t)i * p.bias_ld];
+    };
+    if (tile_ok[0]) load_bias(0, bias_t[0]);
 
     fetch_q(0);
     stash_q(0, 0, kc == 0);
@@ -213,15 +236,10 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
         const int tl = w * TPW + t;            // tile inside the chunk
         const int j0 = (tile0 + tl) * 32;
         if (j0 < S) {                          // wave-uniform
-          const int j = j0 + x;
-          f32x16 z;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int qi = i0 + 16 * g + r;
-            z[r] = (qi < S && j < S) ? biasg[(int64_t)qi * p.bias_ld + j] : 0.0f;
-          }
           const T* krow = Kc + (tl * 32 + x) * L::KSTR;
-          z = mma(qaugA, ld8<T>(krow + DP + 8 * g), z);
+          f32x16 z = mma(qaugA, ld8<T>(krow + DP + 8 * g), bzn);
+          if (t + 1 < TPW && tile_ok[t + 1 < TPW ? t + 1 : 0]) load_bias(it, bias_t[t + 1 < TPW ? t + 1 : 0]);
+          else if (more) load_bias(it + 1, bias_t[0]);
 #pragma unroll
           for (int s = 0; s < KS; ++s) z = mma(qA[s], ld8<T>(krow + (DP / 2) * g + 8 * s), z);
           f32x16 dp = acc_zero();
@@ -230,7 +248,7 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
           f32x16 ds;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float pr = fast_exp2(__builtin_fmaf(z[r], MF_LOG2E, -l2v[r]));
+            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2v[r]));
             z[r] = pr;
             ds[r] = pr * (dp[r] - dlv[r]);
           }
@@ -316,7 +334,10 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
           for (int u = 0; u < 2; ++u) {
             const int d0 = (DP / 2) * g + 16 * dt + 8 * u;
             if (d0 < D) {
-              st8<T>(dKg + (int64_t)j * p.dk.ss + d0, acc_half<T>(dk[t][dt], u));
+              f32x16 dks = dk[t][dt];
+#pragma unroll
+              for (int i = 0; i < 16; ++i) dks[i] *= p.scale;
+              st8<T>(dKg + (int64_t)j * p.dk.ss + d0, acc_half<T>(dks, u));
               st8<T>(dVg + (int64_t)j * p.dv.ss + d0, acc_half<T>(dv[t][dt], u));
             }
           }
@@ -439,6 +460,8 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
   const T* Vg = reinterpret_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
   const float* biasg = p.bias + b * p.bias_sb + h * p.bias_sh;
 
+  const float cexp = p.scale * MF_LOG2E;   // the accumulator holds z / scale
+  const float inv_scale = 1.0f / p.scale;
   // the bias patch is the same for every row n: keep it in registers as the accumulator seed
   f32x16 bz[TR], acc[TR];
 #pragma unroll
@@ -447,7 +470,7 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = (jt0 + t) * 32 + 16 * g + r;
-      bz[t][r] = j < S ? biasg[(int64_t)qi_c * p.bias_ld + j] : 0.0f;
+      bz[t][r] = j < p.bias_ld ? biasg[(int64_t)qi_c * p.bias_ld + j] : 0.0f;
     }
   }
   frag qaug = frag_zero<T>();
@@ -475,14 +498,14 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
     }
     if (tid < ROWS) {
       const int j = jt0 * 32 + tid;
-      mreg = j < S ? load_any(p.mask, p.mask_dtype, b * p.mask_sb + n * p.mask_sn + (int64_t)j * p.mask_sj)
+      mreg = j < S ? load_any(p.mask, p.mask_dtype, b * p.mask_sb + n * p.mask_sn + (int64_t)j * p.mask_sj) * inv_scale
                    : -__builtin_inff();
     }
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d0 = (DP / 2) * g + 8 * s;
       const bool ok = qi < S && d0 < D;
-      qf[s] = ok ? scale8<T>(ld8<T>(Qg + (int64_t)n * p.q.sn + d0), p.scale) : frag_zero<T>();
+      qf[s] = ok ? ld8<T>(Qg + (int64_t)n * p.q.sn + d0) : frag_zero<T>();
       dof[s] = ok ? ld8<T>(dOg + (int64_t)n * p.dO.sn + d0) : frag_zero<T>();
     }
     const int64_t ridx = (((int64_t)b * p.N + n) * p.H + h) * S + qi_c;
@@ -543,7 +566,7 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float pr = fast_exp2(__builtin_fmaf(z[r], MF_LOG2E, -l2c));
+            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2c));
             acc[t][r] = __builtin_fmaf(pr, dp[r] - dlc, acc[t][r]);
           }
         }
@@ -574,7 +597,7 @@ __global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, fl
 }
 
 // Key tiles per wavefront patch: limited by the registers the patch and its bias seed occupy.
-static int dbias_tr(int dtype, int D) { return dtype == MF_F32 ? 1 : (D > 32 ? 2 : 3); }
+static int dbias_tr(int dtype, int D) { (void)D; return dtype == MF_F32 ? 1 : 2; }
 
 int evo_dbias_chunks(int B, int N, int S, int H, int D, int dtype) {
   const int TR = dbias_tr(dtype, D);
@@ -619,7 +642,7 @@ template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const Evo
 
 template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipStream_t stream) {
   constexpr bool wide = sizeof(T) == 4;
-  if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 3>(p, stream);
+  if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 2>(p, stream);
   if (p.D <= 64) return launch_dbias_t<T, 64, wide ? 1 : 2>(p, stream);
   return hipErrorInvalidValue;
 }

@@ -45,35 +45,58 @@ hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t strea
 }
 
 // =================================================================================================
-// weight preparation
+// weight preparation:  W' = gamma (.) W in both layouts, column sums of W', folded bias
 // =================================================================================================
+// One work-group owns 16 columns of W and all K rows: reads and writes of the [K, N] layout are
+// coalesced along n, the transposed [N, KP] copy goes through LDS so its rows are written whole.
 template <typename T>
 __global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= p.N) return;
+  __shared__ float tile[16][257];     // [n][k], K <= 256
+  __shared__ float red_cs[16][17], red_bp[16][17];
+  const int tid = threadIdx.x, nn = tid & 15, kk = tid >> 4;
+  const int n = blockIdx.x * 16 + nn;
   const T* W = reinterpret_cast<const T*>(p.W);
   const T* gamma = reinterpret_cast<const T*>(p.gamma);
   const T* beta = reinterpret_cast<const T*>(p.beta);
   T* Wt = reinterpret_cast<T*>(p.Wt);
   T* Wg = reinterpret_cast<T*>(p.Wg);
   float cs = 0.0f, bp = 0.0f;
-  for (int k = 0; k < p.K; ++k) {
-    const float w = to_f(W[(int64_t)k * p.N + n]);
-    const T gw = (T)(to_f(gamma[k]) * w);
-    if (Wt) Wt[(int64_t)n * p.KP + k] = gw;
-    if (Wg) Wg[(int64_t)k * p.N + n] = gw;
-    cs += to_f(gw);
-    if (beta) bp += to_f(beta[k]) * w;
+  for (int k = kk; k < p.KP; k += 16) {
+    float gwf = 0.0f;
+    if (k < p.K && n < p.N) {
+      const float w = to_f(W[(int64_t)k * p.N + n]);
+      const T gw = (T)(to_f(gamma[k]) * w);
+      if (Wg) Wg[(int64_t)k * p.N + n] = gw;
+      gwf = to_f(gw);
+      cs += gwf;
+      if (beta) bp += to_f(beta[k]) * w;
+    }
+    tile[nn][k] = gwf;
   }
-  if (Wt)
-    for (int k = p.K; k < p.KP; ++k) Wt[(int64_t)n * p.KP + k] = (T)0.0f;
-  if (p.colsum) p.colsum[n] = cs;
-  if (p.bprime) p.bprime[n] = bp + (p.b ? to_f(reinterpret_cast<const T*>(p.b)[n]) : 0.0f);
+  red_cs[nn][kk] = cs;
+  red_bp[nn][kk] = bp;
+  __syncthreads();
+  if (tid < 16) {
+    const int n2 = blockIdx.x * 16 + tid;
+    float a = 0.0f, b2 = 0.0f;
+    for (int j = 0; j < 16; ++j) { a += red_cs[tid][j]; b2 += red_bp[tid][j]; }
+    if (n2 < p.N) {
+      if (p.colsum) p.colsum[n2] = a;
+      if (p.bprime) p.bprime[n2] = b2 + (p.b ? to_f(reinterpret_cast<const T*>(p.b)[n2]) : 0.0f);
+    }
+  }
+  if (Wt) {
+    for (int i = tid; i < 16 * p.KP; i += 256) {
+      const int r = i / p.KP, k = i % p.KP;
+      const int n2 = blockIdx.x * 16 + r;
+      if (n2 < p.N) Wt[(int64_t)n2 * p.KP + k] = (T)tile[r][k];
+    }
+  }
 }
 
 hipError_t launch_ln_prep(const LnParams& p, bool forward, hipStream_t stream) {
   (void)forward;
-  const unsigned blocks = (unsigned)((p.N + 255) / 256);
+  const unsigned blocks = (unsigned)((p.N + 15) / 16);
   switch (p.dtype) {
     case MF_BF16: hipLaunchKernelGGL(ln_prep_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
     case MF_F16: hipLaunchKernelGGL(ln_prep_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, p); break;

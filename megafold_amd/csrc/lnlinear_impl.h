@@ -617,6 +617,35 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
   }
 }
 
+// Sum of the per-range partials in a fixed order.  A work-group owns 64 consecutive float4 groups
+// of the flattened [K, N] matrix; its four 64-thread groups each add a quarter of the ranges and
+// the quarters are combined through LDS.  The result overwrites range 0.  Work-groups past the matrix
+// do the same for the column sums.
+template <typename T>
+__global__ void __launch_bounds__(256) ln_bwd_reduce_kernel(float* __restrict__ Gpart, float* __restrict__ spart,
+                                                            int64_t kn, int N, int R, int g_blocks) {
+  __shared__ f32x4 red[4][64];
+  const int tid = threadIdx.x, c = tid & 63, rg = tid >> 6;
+  if ((int)blockIdx.x < g_blocks) {
+    const int64_t e = ((int64_t)blockIdx.x * 64 + c) * 4;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (e < kn) {
+#pragma unroll 8
+      for (int r = rg; r < R; r += 4) acc += *reinterpret_cast<const f32x4*>(Gpart + (int64_t)r * kn + e);
+    }
+    red[rg][c] = acc;
+    __syncthreads();
+    if (rg == 0 && e < kn) *reinterpret_cast<f32x4*>(Gpart + e) = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+  } else {
+    const int n = ((int)blockIdx.x - g_blocks) * 256 + tid;
+    if (n < N) {
+      float sacc = 0.0f;
+      for (int r = 0; r < R; ++r) sacc += spart[(int64_t)r * N + n];
+      spart[n] = sacc;
+    }
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) {
   const int k = blockIdx.x, tid = threadIdx.x;
@@ -625,11 +654,8 @@ __global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) 
   const float bet = p.beta ? to_f(reinterpret_cast<const T*>(p.beta)[k]) : 0.0f;
   float dg = 0.0f, dbt = 0.0f;
   for (int n = tid; n < p.N; n += 256) {
-    float G = 0.0f, s = 0.0f;
-    for (int r = 0; r < p.R; ++r) {
-      G += p.Gpart[((int64_t)r * p.K + k) * p.N + n];
-      s += p.spart[(int64_t)r * p.N + n];
-    }
+    const float G = p.Gpart[(int64_t)k * p.N + n];
+    const float s = p.spart[n];
     const float wv = to_f(W[(int64_t)k * p.N + n]);
     p.dW[(int64_t)k * p.N + n] = gam * G + bet * s;
     dg += wv * G;
@@ -649,7 +675,6 @@ __global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) 
   }
 }
 
-
 template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, const void* dY, hipStream_t stream) {
   using Sh = DwShape<KP>;
   constexpr int UNIT = 16 / (int)sizeof(T);
@@ -665,6 +690,13 @@ template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, c
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)p.R, (unsigned)gy), dim3(256), smem, stream, p, reinterpret_cast<const T*>(dY));
   hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int64_t kn = (int64_t)p.K * p.N;
+  const int g_blocks = (int)((kn / 4 + 63) / 64);
+  const int s_blocks = (p.N + 255) / 256;
+  hipLaunchKernelGGL(ln_bwd_reduce_kernel<T>, dim3((unsigned)(g_blocks + s_blocks)), dim3(256), 0, stream, p.Gpart, p.spart,
+                     kn, p.N, p.R, g_blocks);
+  e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(ln_bwd_finalize_kernel<T>, dim3((unsigned)p.K), dim3(256), 0, stream, p);
   return hipGetLastError();

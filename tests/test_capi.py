@@ -90,12 +90,9 @@ def test_attention_argument_errors(mutate, code, text):
 def test_attention_workspace_contract():
     lib = _lib.lib()
     a = _evo_args()
-    assert lib.mf_evoattn_fwd_workspace_bytes(C.byref(a)) == 0          # fp32 bias is read in place
-    a.bias_dtype = _lib.MF_BF16
-    need = lib.mf_evoattn_fwd_workspace_bytes(C.byref(a))
+    need = lib.mf_evoattn_fwd_workspace_bytes(C.byref(a))               # fp32 copy of bias / scale
     assert need >= 1 * 2 * 64 * 64 * 4
     assert lib.mf_evoattn_fwd(C.byref(a)) == -6 and "workspace" in lib.mf_last_error().decode()
-    a.bias_dtype = _lib.MF_F32
     for f in ("dO", "dq", "dk", "dv", "dbias"):
         setattr(a, f, 0x10000)
     a.do_stride = a.dq_stride = a.dk_stride = a.dv_stride = a.q_stride
