@@ -55,7 +55,8 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     if not srcs:
         raise RuntimeError("no HIP sources under %s" % CSRC)
     objs = [OBJ / (s.stem + ".o") for s in srcs]
-    cmds = [[hipcc, *HIPCC_FLAGS, "-c", str(s), "-o", str(o)] for s, o in zip(srcs, objs)]
+    extra = os.environ.get("MF_HIPCC_EXTRA", "").split()   # e.g. -DMF_TIMELINE (development builds)
+    cmds = [[hipcc, *HIPCC_FLAGS, *extra, "-c", str(s), "-o", str(o)] for s, o in zip(srcs, objs)]
     jobs = jobs or min(8, len(cmds))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         for cmd, _ in zip(cmds, ex.map(_run, cmds)):

@@ -85,7 +85,6 @@ int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStrea
   p.B = a->B; p.N = a->N; p.S = a->S; p.H = a->H; p.D = a->D;
   p.dtype = a->dtype;
   p.scale = a->scale;
-  { const char* e = getenv("MF_DBG"); p.dbg = e ? atoi(e) : 0; }
   p.q = tens(a->q, a->q_stride); p.k = tens(a->k, a->k_stride); p.v = tens(a->v, a->v_stride);
   p.o = tens(a->o, a->o_stride);
   p.mask = a->mask; p.mask_dtype = a->mask_dtype;
@@ -159,6 +158,10 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   p.delta = reinterpret_cast<float*>(ws + pl.off_delta);
   p.dbias = a->dbias;
   p.n_chunks = pl.n_chunks;
+#ifdef MF_TIMELINE
+  { const char* e = getenv("MF_TL_PTR"); p.tl = e ? reinterpret_cast<unsigned*>(strtoull(e, nullptr, 16)) : nullptr;
+    const char* f = getenv("MF_TL_BLOCK"); p.tl_block = f ? atoi(f) : 0; }
+#endif
   p.rows_per_chunk = pl.rows_per_chunk;
   p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
   const int phases = a->phases == 0 ? (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;

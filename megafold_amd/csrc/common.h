@@ -210,4 +210,110 @@ template <> __device__ __forceinline__ void split_hi_lo<float>(float v, float& h
   lo = 0.0f;
 }
 
+// ---- LDS tile of DP-wide rows ----------------------------------------------------------------------
+// 16-bit element types: rows are stored unpadded (DP*2 bytes) with their 16-byte chunks XOR-swizzled
+// by the row number, which keeps both fragment reads (one row per lane, same chunk) and transposing
+// reads free of bank conflicts and — unlike padding — is compatible with direct global->LDS loads,
+// whose destination is "lane i writes 16 bytes at base + 16*i".  fp32 keeps padded rows and is staged
+// through registers.
+template <typename T, int DP> struct Tile {
+  static constexpr bool kAsync = sizeof(T) == 2;
+  static constexpr int CPR = DP * (int)sizeof(T) / 16;          // 16-byte chunks per row
+  static constexpr int EPC = 16 / (int)sizeof(T);               // elements per chunk
+  static constexpr int RP = CPR >= 8 ? 1 : 8 / CPR;             // rows per 128 bytes
+  static constexpr int STRIDE = kAsync ? DP : DP + 4;           // elements between rows
+  static __device__ __forceinline__ int swz(int row) { return kAsync ? (row / RP) % (CPR < 8 ? CPR : 8) : 0; }
+  // element offset of (row, col); col must not cross a chunk together with the access width
+  static __device__ __forceinline__ int off(int row, int col) {
+    if (kAsync) return row * DP + ((((col / EPC) ^ swz(row))) * EPC) + (col % EPC);
+    return row * STRIDE + col;
+  }
+  // the 8 values X[k0 + 8*g + e][own_col], e = 0..7 (see TrRead for the lane protocol)
+  static __device__ __forceinline__ frag_t<T> tr_read(const T* tile, int k0, int g, int l, int chunk_col, int own_col) {
+    if constexpr (kAsync) {
+      const int a = (l >> 2) & 3;
+      const int r0 = k0 + 8 * g + a, r1 = r0 + 4;
+      const T* p0 = tile + off(r0, chunk_col);
+      const T* p1 = tile + off(r1, chunk_col);
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      s16x8 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+      return __builtin_bit_cast(frag_t<T>, v);
+    } else {
+      frag_t<T> v;
+      const T* p = tile + (k0 + 8 * g) * STRIDE + own_col;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = p[e * STRIDE];
+      return v;
+    }
+  }
+};
+
+// Direct global->LDS copy of 16 bytes per lane: lane i's data lands at lds_base + 16*i (lds_base must
+// be wave-uniform).  Completion is tracked by vmcnt like any vector memory load.
+__device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+}
+// Work-group barrier without the memory fence __syncthreads() implies (which would drain every
+// outstanding direct-to-LDS load): wait for this wavefront's LDS traffic and all but the newest
+// `VM` vector-memory operations, then synchronise.
+template <int VM> __device__ __forceinline__ void barrier_keep_vm() {
+  static_assert(VM >= 0 && VM < 64, "vmcnt range");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(((VM & 15) | ((VM >> 4) << 14)) | (7 << 4) | (0 << 8));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// ---- carrier fragments: scalars riding through one extra MFMA contraction step -------------------
+// 16-bit types: a 32-bit word holds two slots (value split as hi + lo, or the pair (1, 1)); a carrier
+// fragment is {w0, w1, 0, 0} = slots (w0.lo, w0.hi, w1.lo, w1.hi, 0, 0, 0, 0).  fp32: a word is one
+// slot, the fragment is {w0, w1, 0, ...}.  Pairing A = {ones, -x} with B = {y, ones} adds y - x to
+// every element of the tile exactly (to ~2^-17 relative for the split 16-bit values).
+template <typename T> __device__ __forceinline__ frag_t<T> make_aug(unsigned w0, unsigned w1) {
+  u32x4 v = {w0, w1, 0u, 0u};
+  return __builtin_bit_cast(frag_t<T>, v);
+}
+template <> __device__ __forceinline__ f32x8 make_aug<float>(unsigned w0, unsigned w1) {
+  f32x8 f = {__builtin_bit_cast(float, w0), __builtin_bit_cast(float, w1), 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  return f;
+}
+template <typename T> __device__ __forceinline__ unsigned pack_split(float m) {
+  T hi, lo;
+  split_hi_lo<T>(m, hi, lo);
+  typedef T pair_t __attribute__((ext_vector_type(2)));
+  pair_t pr = {hi, lo};
+  return __builtin_bit_cast(unsigned, pr);
+}
+template <> __device__ __forceinline__ unsigned pack_split<float>(float m) { return __builtin_bit_cast(unsigned, m); }
+template <typename T> __device__ __forceinline__ unsigned ones_word() {
+  typedef T pair_t __attribute__((ext_vector_type(2)));
+  pair_t pr = {(T)1.0f, (T)1.0f};
+  return __builtin_bit_cast(unsigned, pr);
+}
+template <> __device__ __forceinline__ unsigned ones_word<float>() { return __builtin_bit_cast(unsigned, 1.0f); }
+
 }  // namespace mf
+
+// Force a value to be computed where this statement stands.  The optimiser otherwise sinks arithmetic
+// on loaded registers towards its first use, which can carry it past the issue of the NEXT batch of
+// loads: the in-order vector-memory counter then makes the old value wait for the new loads.
+template <typename V> __device__ __forceinline__ void pin(V& v) { asm volatile("" : "+v"(v)); }
+
+// ---- development aid: per-phase cycle stamps ------------------------------------------------------
+// Compiled in only with -DMF_TIMELINE.  MF_TL(p, slot) makes lane 0 of every wavefront of the chosen
+// work-group store the shader clock at p.tl[slot]; the caller supplies the buffer address through the
+// environment variable MF_TL_PTR (hex) and the work-group through MF_TL_BLOCK.
+#ifdef MF_TIMELINE
+#define MF_TL(p, slot)                                                                              \
+  do {                                                                                              \
+    if ((p).tl && (int)blockIdx.x == (p).tl_block && (threadIdx.x & 63) == 0)                       \
+      (p).tl[(slot)] = (unsigned)__builtin_readcyclecounter();                                      \
+  } while (0)
+#else
+#define MF_TL(p, slot) do { } while (0)
+#endif

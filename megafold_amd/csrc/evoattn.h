@@ -35,7 +35,10 @@ struct EvoParams {
   float* delta;    // [B, N, H, S] fp32 rowsum(dO * O)
   float* dbias;    // [B, H, S, S] fp32 or nullptr
   float* dbias_part;  // [n_chunks, B, H, S, S] fp32 partial sums (nullptr when n_chunks == 1)
-  int dbg;         // experiment switches (0 in production)
+#ifdef MF_TIMELINE
+  unsigned* tl;    // development aid: cycle stamps of one work-group (see MF_TL in common.h)
+  int tl_block;
+#endif
   int n_chunks;    // number of N-chunks the bias-gradient kernel splits the rows into
   int rows_per_chunk;
 };

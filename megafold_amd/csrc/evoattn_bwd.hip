@@ -24,19 +24,29 @@ namespace mf {
 template <typename T, int DP> struct BwdLayout {
   static constexpr int UNIT = 16 / (int)sizeof(T);
   static constexpr int KRAW = DP + 16;
-  static constexpr int KSTR = ((KRAW / UNIT) % 2 == 0) ? KRAW + UNIT : KRAW;   // K rows + mask carrier
-  static constexpr int QSTR = ((DP / UNIT) % 2 == 0) ? DP + UNIT : DP;         // Q / dO / V rows
+  static constexpr int KSTR = ((KRAW / UNIT) % 2 == 0) ? KRAW + UNIT : KRAW;   // K rows + mask carrier (dBias kernel)
+  static constexpr int QSTR = ((DP / UNIT) % 2 == 0) ? DP + UNIT : DP;         // K / Q / dO / V rows
   static constexpr int TSTR = ((32 / UNIT) % 2 == 0) ? 32 + UNIT : 32;         // dS tile rows
   static constexpr int SSTR = DP + 4;                                          // fp32 dQ slab rows
   static constexpr int TR_BYTES = 32 * TSTR * (int)sizeof(T);
   static constexpr int SLAB_BYTES = 32 * SSTR * 4;
-  static constexpr int WAVE_BYTES = TR_BYTES > SLAB_BYTES ? TR_BYTES : SLAB_BYTES;  // per-wave scratch (aliased)
+  // per-wavefront scratch: one dS tile per key tile of the wavefront, aliased with its dQ slab
+  static constexpr int wave_bytes(int tpw) { return tpw * TR_BYTES > SLAB_BYTES ? tpw * TR_BYTES : SLAB_BYTES; }
   static constexpr int STAGE_ELEMS = 2 * 32 * QSTR;                            // Q tile + dO tile
 };
 
 // =================================================================================================
 // dQ, dK, dV (+ delta)
 // =================================================================================================
+// Per (query tile, key tile) step, with everything additive riding through carrier MFMA steps:
+//   z' = <q, k> + bias/s + mask/s - LSE/s      (5 = 1 carrier + DP/16 MFMAs for D = 32: 3)
+//   P  = exp2(c z'),  c = s log2 e
+//   d' = <dO, v> - delta                        (1 carrier + DP/16 MFMAs)
+//   dS = P d'
+//   dV += P^T dO,  dK += dS^T Q  (operands: P, dS straight from the accumulator registers; dO^T, Q^T
+//        through transposing LDS reads),  dQ += dS K (dS through a per-wavefront LDS tile, K^T through
+//        transposing reads)
+// so the vector ALU does one multiply, one exp2, one multiply and two packed converts per logit.
 template <typename T, int DP, int TPW, int MAXT>
 __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   using L = BwdLayout<T, DP>;
@@ -49,11 +59,12 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   const int KC = NW * TPW * 32;                  // keys per chunk
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T* Kc = reinterpret_cast<T*>(smem_raw);                                   // [KC][KSTR]
-  T* Stage = Kc + KC * L::KSTR;                                             // [2][Q tile | dO tile]
-  float* Lv = reinterpret_cast<float*>(Stage + 2 * L::STAGE_ELEMS);         // [2][32] LSE * log2(e)
-  float* Dv = Lv + 64;                                                      // [2][32] delta
-  unsigned char* Wv = reinterpret_cast<unsigned char*>(Dv + 64);            // [NW][WAVE_BYTES]
+  T* Kc = reinterpret_cast<T*>(smem_raw);                                   // [KC][QSTR]
+  T* Stage = Kc + KC * L::QSTR;                                             // [2][Q tile | dO tile]
+  unsigned* Lpk = reinterpret_cast<unsigned*>(Stage + 2 * L::STAGE_ELEMS);  // [2][32] packed -LSE/scale
+  unsigned* Dpk = Lpk + 64;                                                 // [2][32] packed -delta
+  unsigned char* Wv = reinterpret_cast<unsigned char*>(Dpk + 64);           // [NW][WAVE_BYTES]
+  constexpr int WAVE_BYTES = L::wave_bytes(TPW);
 
   const int bid = blockIdx.x;
   const int xcd = bid & 7, kq = bid >> 3;
@@ -65,6 +76,8 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int S = p.S, D = p.D;
   const int NT = (S + 31) >> 5;
+  const float cexp = p.scale * MF_LOG2E;   // the accumulator holds z / scale
+  const float inv_scale = 1.0f / p.scale;
 
   const T* Qg = reinterpret_cast<const T*>(p.q.ptr) + b * p.q.sb + n * p.q.sn + h * p.q.sh;
   const T* Kg = reinterpret_cast<const T*>(p.k.ptr) + b * p.k.sb + n * p.k.sn + h * p.k.sh;
@@ -78,44 +91,38 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   const int64_t mask_base = b * p.mask_sb + n * p.mask_sn;
   const int64_t row_base = (((int64_t)b * p.N + n) * p.H + h) * S;   // into lse / delta
 
-  T* Trw = reinterpret_cast<T*>(Wv + w * L::WAVE_BYTES);
-  float* Slw = reinterpret_cast<float*>(Wv + w * L::WAVE_BYTES);
+  T* Trw = reinterpret_cast<T*>(Wv + w * WAVE_BYTES);
+  float* Slw = reinterpret_cast<float*>(Wv + w * WAVE_BYTES);
 
-  frag qaugA = frag_zero<T>();   // Q side of the mask-carrier step (A operand here)
-  if (g == 0) { qaugA[0] = (T)1.0f; qaugA[1] = (T)1.0f; }
+  const unsigned ones_g = g == 0 ? ones_word<T>() : 0u;     // carrier slots live in the lower lane half only
+  const frag vaugB = make_aug<T>(ones_g, 0u);                // B side of the delta carrier
 
-  const float cexp = p.scale * MF_LOG2E;   // the accumulator holds z / scale (unscaled q.k + bias/scale + mask/scale)
-  const float inv_scale = 1.0f / p.scale;
-
-  // ---- staging of one query tile: Q, dO, LSE, delta --------------------------------------------
+  // ---- staging of one query tile: Q, dO, packed -LSE/scale and -delta ----------------------------
+  // Rows past S are clamped for the loads; their LSE is +inf, which makes every probability exactly 0.
   frag sq[PF], sdo[PF];
-  float sdelta[PF], slse[PF];
+  float sdelta[PF], sls[PF];
   auto fetch_q = [&](int it) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int item = tid + i * nthr;
-      sdelta[i] = 0.0f; slse[i] = __builtin_inff();
-      sq[i] = frag_zero<T>(); sdo[i] = frag_zero<T>();
       if (item < QITEMS) {
         const int row = item / CPR, dc = item % CPR;
         const int qi = it * 32 + row;
-        const bool ok = qi < S && 8 * dc < D;
-        frag of = frag_zero<T>();
-        if (ok) {
-          sq[i] = ld8<T>(Qg + (int64_t)qi * p.q.ss + 8 * dc);
-          sdo[i] = ld8<T>(dOg + (int64_t)qi * p.dO.ss + 8 * dc);
-          of = ld8<T>(Og + (int64_t)qi * p.o.ss + 8 * dc);
-        }
+        const int qc = qi < S ? qi : S - 1;
+        const bool dok = 8 * dc < D;
+        sq[i] = dok ? ld8<T>(Qg + (int64_t)qc * p.q.ss + 8 * dc) : frag_zero<T>();
+        sdo[i] = dok ? ld8<T>(dOg + (int64_t)qc * p.dO.ss + 8 * dc) : frag_zero<T>();
+        const frag of = dok ? ld8<T>(Og + (int64_t)qc * p.o.ss + 8 * dc) : frag_zero<T>();
         float part = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) part += (float)sdo[i][e] * (float)of[e];
 #pragma unroll
         for (int m = 1; m < CPR; m <<= 1) part += __shfl_xor(part, m);
         sdelta[i] = part;
+        sls[i] = __builtin_inff();
         if (dc == 0 && qi < S) {
           const float lse = p.lse[row_base + qi];
-          // fully masked row: LSE = -inf; +inf makes every recomputed probability exactly 0
-          slse[i] = (lse == -__builtin_inff()) ? __builtin_inff() : lse * MF_LOG2E;
+          sls[i] = (lse == -__builtin_inff()) ? __builtin_inff() : lse * inv_scale;
         }
       }
     }
@@ -131,8 +138,8 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
         st8<T>(qd + row * L::QSTR + 8 * dc, sq[i]);
         st8<T>(dod + row * L::QSTR + 8 * dc, sdo[i]);
         if (dc == 0) {
-          Lv[buf * 32 + row] = slse[i];
-          Dv[buf * 32 + row] = sdelta[i];
+          Lpk[buf * 32 + row] = pack_split<T>(-sls[i]);
+          Dpk[buf * 32 + row] = pack_split<T>(-sdelta[i]);
           const int qi = it * 32 + row;
           if (write_delta && qi < S) p.delta[row_base + qi] = sdelta[i];
         }
@@ -143,34 +150,34 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   const int nchunks = (NT + NW * TPW - 1) / (NW * TPW);
   for (int kc = 0; kc < nchunks; ++kc) {
     const int tile0 = kc * NW * TPW;
-    // ---- stage this chunk's K rows (plain order) with the mask carrier columns ------------------
+    // ---- stage this chunk's K rows (keys past S clamped: their mask is -inf) ----------------------
     for (int c = tid; c < KC * CPR; c += nthr) {
       const int kk = c / CPR, dc = c % CPR;
-      const int j = tile0 * 32 + kk;
-      const bool ok = j < S && 8 * dc < D;
-      st8<T>(Kc + kk * L::KSTR + 8 * dc, ok ? ld8<T>(Kg + (int64_t)j * p.k.ss + 8 * dc) : frag_zero<T>());
+      int j = tile0 * 32 + kk;
+      j = j < S ? j : S - 1;
+      st8<T>(Kc + kk * L::QSTR + 8 * dc, 8 * dc < D ? ld8<T>(Kg + (int64_t)j * p.k.ss + 8 * dc) : frag_zero<T>());
     }
-    for (int kk = tid; kk < KC; kk += nthr) {
-      const int j = tile0 * 32 + kk;
-      const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) * inv_scale
-                             : -__builtin_inff();
-      frag a = frag_zero<T>();
-      T hi, lo;
-      split_hi_lo<T>(mv, hi, lo);
-      a[0] = hi; a[1] = lo;
-      st8<T>(Kc + kk * L::KSTR + DP, a);
-      st8<T>(Kc + kk * L::KSTR + DP + 8, frag_zero<T>());
-    }
-    // V fragments of this wavefront's tiles (B operand of dP = dO V^T): lane (x, g) <-> key j0 + x
+    // this wavefront's key tiles: V fragments (B operand of dO V^T), packed mask/scale, bias pointers
     frag vf[TPW][KS];
+    unsigned mk[TPW];
+    const float* bias_t[TPW];
+    bool tile_ok[TPW];
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-      const int j = (tile0 + w * TPW + t) * 32 + x;
+      const int j0 = (tile0 + w * TPW + t) * 32;
+      const int j = j0 + x;
+      const int jc = j < S ? j : S - 1;
+      tile_ok[t] = j0 < S;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const int d0 = (DP / 2) * g + 8 * s;
-        vf[t][s] = (j < S && d0 < D) ? ld8<T>(Vg + (int64_t)j * p.v.ss + d0) : frag_zero<T>();
+        vf[t][s] = d0 < D ? ld8<T>(Vg + (int64_t)jc * p.v.ss + d0) : frag_zero<T>();
       }
+      const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) * inv_scale
+                             : -__builtin_inff();
+      mk[t] = g == 0 ? pack_split<T>(mv) : 0u;
+      // bias/scale copy is zero padded to whole tiles: register i of half g <-> query 32*it + 16*g + i
+      bias_t[t] = biasg + (int64_t)(16 * g) * p.bias_ld + (tile_ok[t] ? j0 : 0) + x;
     }
     f32x16 dk[TPW][DT], dv[TPW][DT];
 #pragma unroll
@@ -178,24 +185,14 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) { dk[t][dt] = acc_zero(); dv[t][dt] = acc_zero(); }
 
-    // bias/scale tile of the next (query tile, key tile) step, loaded one step ahead.  The copy in
-    // the workspace is zero padded to whole tiles, so no bounds checks: register i of half g <->
-    // query 32*it + 16*g + i, lane x <-> key j0 + x.
-    const float* bias_t[TPW];
-    bool tile_ok[TPW];
-#pragma unroll
-    for (int t = 0; t < TPW; ++t) {
-      const int j0 = (tile0 + w * TPW + t) * 32;
-      tile_ok[t] = j0 < S;
-      bias_t[t] = biasg + (int64_t)(16 * g) * p.bias_ld + (tile_ok[t] ? j0 : 0) + x;
-    }
+    // bias/scale tile of the next (query tile, key tile) step, loaded one step ahead
     f32x16 bzn;
     auto load_bias = [&](int it, const float* base) {
       const float* bp = base + (int64_t)it * 32 * p.bias_ld;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) bzn[i] = bp[(int64_t)i * p.bias_ld];
+      for (int i = 0; i < 16; ++i) bzn[i] = bp[i * (int)p.bias_ld];
     };
-    if (tile_ok[0]) load_bias(0, bias_t[0]);
+    load_bias(0, bias_t[0]);   // idle tile slots read (and ignore) column block 0
 
     fetch_q(0);
     stash_q(0, 0, kc == 0);
@@ -210,23 +207,18 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
       const T* dos = qs + 32 * L::QSTR;
       const int i0 = it * 32;
 
-      // per-register row constants: register r of half g <-> query i0 + 16*g + r
-      float l2v[16], dlv[16];
-#pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4) {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(Lv + buf * 32 + 16 * g + 4 * c4);
-        const f32x4 d = *reinterpret_cast<const f32x4*>(Dv + buf * 32 + 16 * g + 4 * c4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) { l2v[4 * c4 + e] = a[e]; dlv[4 * c4 + e] = d[e]; }
-      }
-      // A operands of S = Q K^T and dP = dO V^T: operand row x holds tile row unperm32(x)
-      frag qA[KS], doA[KS];
+      // A operands of S = Q K^T and dP = dO V^T: operand row x holds tile row unperm32(x), so that
+      // accumulator register i of half g belongs to query i0 + 16*g + i
       const int arow = unperm32(x);
+      frag qA[KS], doA[KS];
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         qA[s] = ld8<T>(qs + arow * L::QSTR + (DP / 2) * g + 8 * s);
         doA[s] = ld8<T>(dos + arow * L::QSTR + (DP / 2) * g + 8 * s);
       }
+      const frag qaugA = make_aug<T>(ones_g, g == 0 ? Lpk[buf * 32 + arow] : 0u);
+      const frag doaugA = make_aug<T>(g == 0 ? Dpk[buf * 32 + arow] : 0u, 0u);
+
       f32x16 dq[DT];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) dq[dt] = acc_zero();
@@ -234,23 +226,22 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
 #pragma unroll
       for (int t = 0; t < TPW; ++t) {
         const int tl = w * TPW + t;            // tile inside the chunk
-        const int j0 = (tile0 + tl) * 32;
-        if (j0 < S) {                          // wave-uniform
-          const T* krow = Kc + (tl * 32 + x) * L::KSTR;
-          f32x16 z = mma(qaugA, ld8<T>(krow + DP + 8 * g), bzn);
+        {   // key tiles past S run on clamped keys with mask -inf: they contribute exact zeros
+          const T* krow = Kc + (tl * 32 + x) * L::QSTR;
+          f32x16 z = mma(qaugA, make_aug<T>(mk[t], ones_g), bzn);
           if (t + 1 < TPW && tile_ok[t + 1 < TPW ? t + 1 : 0]) load_bias(it, bias_t[t + 1 < TPW ? t + 1 : 0]);
           else if (more) load_bias(it + 1, bias_t[0]);
 #pragma unroll
           for (int s = 0; s < KS; ++s) z = mma(qA[s], ld8<T>(krow + (DP / 2) * g + 8 * s), z);
-          f32x16 dp = acc_zero();
+          f32x16 dp = mma(doaugA, vaugB, acc_zero());
 #pragma unroll
           for (int s = 0; s < KS; ++s) dp = mma(doA[s], vf[t][s], dp);
           f32x16 ds;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2v[r]));
-            z[r] = pr;
-            ds[r] = pr * (dp[r] - dlv[r]);
+          for (int i = 0; i < 16; ++i) {
+            const float pr = fast_exp2(z[i] * cexp);
+            z[i] = pr;
+            ds[i] = pr * dp[i];
           }
           frag dsf[2];
 #pragma unroll
@@ -265,24 +256,22 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
               dk[t][dt] = mma(qT, dsf[u], dk[t][dt]);
             }
           }
-          // dS tile, rows = keys, through this wavefront's LDS scratch, read back transposed
-          st8<T>(Trw + x * L::TSTR + 16 * g, dsf[0]);
-          st8<T>(Trw + x * L::TSTR + 16 * g + 8, dsf[1]);
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          // dS tile, rows = keys, through this wavefront's LDS scratch (one tile per t, so the tiles of
+          // a query step do not serialise on it), read back transposed.  LDS operations of one
+          // wavefront execute in program order, which is all the ordering this exchange needs.
+          T* trt = Trw + t * 32 * L::TSTR;
+          st8<T>(trt + x * L::TSTR + 16 * g, dsf[0]);
+          st8<T>(trt + x * L::TSTR + 16 * g + 8, dsf[1]);
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
-            const frag dsT = TrRead<T>::read(Trw, L::TSTR, 8 * u + 8 * g, g, l, plain_chunk(l), x);
+            const frag dsT = TrRead<T>::read(trt, L::TSTR, 8 * u + 8 * g, g, l, plain_chunk(l), x);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-              const frag kT = TrRead<T>::read(Kc, L::KSTR, tl * 32 + 8 * u + 8 * g, g, l, dsel_chunk<DP>(dt, l),
+              const frag kT = TrRead<T>::read(Kc, L::QSTR, tl * 32 + 8 * u + 8 * g, g, l, dsel_chunk<DP>(dt, l),
                                               dsel<DP>(dt, x));
               dq[dt] = mma(kT, dsT, dq[dt]);
             }
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
         }
       }
 
@@ -296,14 +285,14 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
           *reinterpret_cast<f32x4*>(Slw + x * L::SSTR + (DP / 2) * g + 16 * dt + 4 * c4) = v;
         }
       if (more) stash_q(it + 1, buf ^ 1, kc == 0);
-      __syncthreads();
+      barrier_keep_vm<63>();   // LDS hand-over only: global loads / stores stay in flight
 
       // fixed-order sum of the NW slabs, scale, store (or add to what earlier key chunks stored)
       for (int item = tid; item < 8 * DP; item += nthr) {
         const int row = item / (DP / 4), c4 = item % (DP / 4);
         f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
         for (int ww = 0; ww < NW; ++ww) {
-          const float* sl = reinterpret_cast<const float*>(Wv + ww * L::WAVE_BYTES);
+          const float* sl = reinterpret_cast<const float*>(Wv + ww * WAVE_BYTES);
           sum += *reinterpret_cast<const f32x4*>(sl + row * L::SSTR + 4 * c4);
         }
         const int qi = i0 + row;
@@ -316,11 +305,12 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) o4[e] += (float)dst[e];
           }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) dst[e] = (T)o4[e];
+          typedef T out4_t __attribute__((ext_vector_type(4)));
+          out4_t ov = {(T)o4[0], (T)o4[1], (T)o4[2], (T)o4[3]};
+          *reinterpret_cast<out4_t*>(dst) = ov;
         }
       }
-      __syncthreads();
+      barrier_keep_vm<63>();
     }
 
     // ---- dK, dV of this wavefront's tiles: lane (x = key, g) owns DP/2 contiguous columns --------
@@ -346,10 +336,337 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// Variant for the 16-bit element types and D <= 32 (the configurations training runs on): one key tile
+// per wavefront, whose K, K^T and V fragments stay in registers for the whole walk over the query
+// tiles, so that the only LDS round trip on a step's critical path is the transposition of dS.  The
+// query-tile operands (Q, dO, Q^T, dO^T) are read at the top of the step, before the matrix products
+// that hide their latency.  The per-wavefront partial dQ goes to one of two alternating fp32 slabs,
+// which leaves ONE work-group barrier per step: the fixed-order sum of the slabs of step `it` runs
+// after that barrier while faster wavefronts already work on step it + 1.
+template <typename T> struct RkLayout {
+  using L = BwdLayout<T, 32>;
+  static constexpr int WAVE_BYTES = L::TR_BYTES + 2 * L::SLAB_BYTES;
+  static size_t smem(int NW) {
+    return (size_t)NW * 32 * L::QSTR * sizeof(T) + (size_t)2 * L::STAGE_ELEMS * sizeof(T) + 128 * 4 +
+           (size_t)NW * WAVE_BYTES;
+  }
+};
+
+template <typename T, int MAXT, int MINW>
+__global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoParams p) {
+  constexpr int DP = 32, KS = 2, CPR = 4, QITEMS = 128;
+  using L = BwdLayout<T, DP>;
+  using frag = frag_t<T>;
+  static_assert(sizeof(T) == 2, "16-bit element types only");
+
+  const int nthr = blockDim.x, NW = nthr >> 6;
+  const int KC = NW * 32;
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* Kc = reinterpret_cast<T*>(smem_raw);                                   // [KC][QSTR]
+  T* Stage = Kc + KC * L::QSTR;                                             // [2][Q tile | dO tile]
+  unsigned* Lpk = reinterpret_cast<unsigned*>(Stage + 2 * L::STAGE_ELEMS);  // [2][32] packed -LSE/scale
+  unsigned* Dpk = Lpk + 64;                                                 // [2][32] packed -delta
+  unsigned char* Wv = reinterpret_cast<unsigned char*>(Dpk + 64);           // [NW][WAVE_BYTES]
+  constexpr int WAVE_BYTES = RkLayout<T>::WAVE_BYTES;
+
+  const int bid = blockIdx.x;
+  const int xcd = bid & 7, kq = bid >> 3;
+  const int bn = (kq / p.H) * 8 + xcd;
+  if (bn >= p.B * p.N) return;
+  const int h = kq % p.H;
+  const int b = bn / p.N, n = bn % p.N;
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const int S = p.S, D = p.D;
+  const int NT = (S + 31) >> 5;
+  const float cexp = p.scale * MF_LOG2E;
+  const float inv_scale = 1.0f / p.scale;
+
+  const T* Qg = reinterpret_cast<const T*>(p.q.ptr) + b * p.q.sb + n * p.q.sn + h * p.q.sh;
+  const T* Kg = reinterpret_cast<const T*>(p.k.ptr) + b * p.k.sb + n * p.k.sn + h * p.k.sh;
+  const T* Vg = reinterpret_cast<const T*>(p.v.ptr) + b * p.v.sb + n * p.v.sn + h * p.v.sh;
+  const T* Og = reinterpret_cast<const T*>(p.o.ptr) + b * p.o.sb + n * p.o.sn + h * p.o.sh;
+  const T* dOg = reinterpret_cast<const T*>(p.dO.ptr) + b * p.dO.sb + n * p.dO.sn + h * p.dO.sh;
+  T* dQg = reinterpret_cast<T*>(p.dq.ptr) + b * p.dq.sb + n * p.dq.sn + h * p.dq.sh;
+  T* dKg = reinterpret_cast<T*>(p.dk.ptr) + b * p.dk.sb + n * p.dk.sn + h * p.dk.sh;
+  T* dVg = reinterpret_cast<T*>(p.dv.ptr) + b * p.dv.sb + n * p.dv.sn + h * p.dv.sh;
+  const float* biasg = p.bias + b * p.bias_sb + h * p.bias_sh;
+  const int64_t mask_base = b * p.mask_sb + n * p.mask_sn;
+  const int64_t row_base = (((int64_t)b * p.N + n) * p.H + h) * S;
+
+  T* Trw = reinterpret_cast<T*>(Wv + w * WAVE_BYTES);
+  float* Slw = reinterpret_cast<float*>(Wv + w * WAVE_BYTES + L::TR_BYTES);   // [2][32][SSTR]
+
+  const unsigned ones_g = g == 0 ? ones_word<T>() : 0u;
+  const frag vaugB = make_aug<T>(ones_g, 0u);
+
+  // Staging of one query tile, split over two groups of 128 threads (one 8-element chunk of one row
+  // each): group A moves Q and -LSE/scale, group B moves dO and forms delta = <dO, O>.  The loads are
+  // issued one step ahead; nothing touches the loaded registers before the stash at the end of the
+  // step, so their latency stays hidden behind the step's matrix products.
+  frag sa, sb;
+  float sls = 0.0f;
+  const int sgrp = tid >> 7;                    // 0: Q, 1: dO / O, >= 2: no staging work
+  const int srow = (tid & 127) / CPR, sdc = tid % CPR;
+  // fetch_q only ISSUES loads (clamped addresses, no arithmetic on the results): zeroing of padded
+  // columns / rows and all conversions happen in stash_q, one step later.
+  const int sd0 = 8 * sdc < D ? 8 * sdc : 0;
+  auto fetch_q = [&](int it) {
+    const int qi = it * 32 + srow;
+    const int qc = qi < S ? qi : S - 1;
+    if (sgrp == 0) {
+      sa = ld8<T>(Qg + (int64_t)qc * p.q.ss + sd0);
+      sls = p.lse[row_base + qc];
+    } else if (sgrp == 1) {
+      sa = ld8<T>(dOg + (int64_t)qc * p.dO.ss + sd0);
+      sb = ld8<T>(Og + (int64_t)qc * p.o.ss + sd0);
+    }
+  };
+  auto stash_q = [&](int it, int buf, bool write_delta) {
+    T* qd = Stage + buf * L::STAGE_ELEMS;
+    const int qi = it * 32 + srow;
+    const bool dok = 8 * sdc < D;
+    if (sgrp == 0) {
+      st8<T>(qd + srow * L::QSTR + 8 * sdc, dok ? sa : frag_zero<T>());
+      if (sdc == 0) {
+        // rows past S and fully masked rows (LSE = -inf) get +inf: every probability becomes exactly 0
+        const float ls = (qi >= S || sls == -__builtin_inff()) ? __builtin_inff() : sls * inv_scale;
+        Lpk[buf * 32 + srow] = pack_split<T>(-ls);
+      }
+    } else if (sgrp == 1) {
+      st8<T>(qd + 32 * L::QSTR + srow * L::QSTR + 8 * sdc, dok ? sa : frag_zero<T>());
+      float part = 0.0f;
+      if (dok) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part += (float)sa[e] * (float)sb[e];
+      }
+#pragma unroll
+      for (int m = 1; m < CPR; m <<= 1) part += __shfl_xor(part, m);
+      if (sdc == 0) {
+        Dpk[buf * 32 + srow] = pack_split<T>(-part);
+        if (write_delta && qi < S) p.delta[row_base + qi] = part;
+      }
+    }
+  };
+
+  const int nchunks = (NT + NW - 1) / NW;
+  for (int kc = 0; kc < nchunks; ++kc) {
+    const int tile0 = kc * NW;
+    for (int c = tid; c < KC * CPR; c += nthr) {
+      const int kk = c / CPR, dc = c % CPR;
+      int j = tile0 * 32 + kk;
+      j = j < S ? j : S - 1;
+      st8<T>(Kc + kk * L::QSTR + 8 * dc, 8 * dc < D ? ld8<T>(Kg + (int64_t)j * p.k.ss + 8 * dc) : frag_zero<T>());
+    }
+    // this wavefront's key tile.  Tiles past S run on clamped keys with mask -inf: exact zeros.
+    const int j0 = (tile0 + w) * 32;
+    const int j = j0 + x;
+    const int jc = j < S ? j : S - 1;
+    frag vf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int d0 = 16 * g + 8 * s;
+      vf[s] = d0 < D ? ld8<T>(Vg + (int64_t)jc * p.v.ss + d0) : frag_zero<T>();
+    }
+    const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) * inv_scale
+                           : -__builtin_inff();
+    const frag maugB = make_aug<T>(g == 0 ? pack_split<T>(mv) : 0u, ones_g);
+    // bias/scale copy is zero padded to whole tiles: register i of half g <-> query 32*it + 16*g + i
+    const float* bias_t = biasg + (int64_t)(16 * g) * p.bias_ld + (j0 < S ? j0 : 0) + x;
+    f32x16 bzn;
+    auto load_bias = [&](int it) {
+      const float* bp = bias_t + (int64_t)it * 32 * p.bias_ld;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bzn[i] = bp[i * (int)p.bias_ld];
+    };
+    load_bias(0);
+
+    fetch_q(0);
+    stash_q(0, 0, kc == 0);
+    __syncthreads();
+
+    frag kf[KS], kT[2];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) kf[s] = ld8<T>(Kc + (w * 32 + x) * L::QSTR + 16 * g + 8 * s);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      kT[u] = TrRead<T>::read(Kc, L::QSTR, w * 32 + 8 * u + 8 * g, g, l, dsel_chunk<DP>(0, l), dsel<DP>(0, x));
+
+    f32x16 dk = acc_zero(), dv = acc_zero();
+
+    // Fixed-order sum of the NW slabs of step `it`, scale, store (or add to what earlier key chunks
+    // stored).  Runs one step late, after the loads of the following step have been requested, so
+    // that neither its LDS reads nor its global store sit on the critical path; for the same reason
+    // the earlier chunks' dQ values are requested a step ahead (fetch_dq_old).
+    typedef T out4_t __attribute__((ext_vector_type(4)));
+    const int rrow = tid >> 3, rc4 = tid & 7;           // threads 0..255: one 4-column run of one row
+    const bool reducer = tid < 8 * DP;
+    out4_t dq_old = {(T)0.0f, (T)0.0f, (T)0.0f, (T)0.0f};
+    auto fetch_dq_old = [&](int it) {
+      if (kc > 0 && reducer) {
+        const int qi = it * 32 + rrow;
+        dq_old = *reinterpret_cast<const out4_t*>(dQg + (int64_t)(qi < S ? qi : S - 1) * p.dq.ss + (4 * rc4 < D ? 4 * rc4 : 0));
+      }
+    };
+    auto reduce_dq = [&](int it) {
+      if (reducer) {
+        const float* sl0 = reinterpret_cast<const float*>(Wv + L::TR_BYTES) + (it & 1) * (32 * L::SSTR) + rrow * L::SSTR + 4 * rc4;
+        f32x4 part[4];     // NW >= 4: the first four reads are unconditional and issued together
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) part[ww] = *reinterpret_cast<const f32x4*>(sl0 + ww * (WAVE_BYTES / 4));
+        f32x4 sum = part[0];
+#pragma unroll
+        for (int ww = 1; ww < 4; ++ww) sum += part[ww];
+        for (int ww = 4; ww < NW; ++ww) sum += *reinterpret_cast<const f32x4*>(sl0 + ww * (WAVE_BYTES / 4));
+        const int qi = it * 32 + rrow;
+        if (qi < S && 4 * rc4 < D) {
+          float o4[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o4[e] = sum[e] * p.scale;
+          if (kc > 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o4[e] += (float)dq_old[e];
+          }
+          out4_t ov = {(T)o4[0], (T)o4[1], (T)o4[2], (T)o4[3]};
+          *reinterpret_cast<out4_t*>(dQg + (int64_t)qi * p.dq.ss + 4 * rc4) = ov;
+        }
+      }
+    };
+
+    for (int it = 0; it < NT; ++it) {
+      const int buf = it & 1;
+      const bool more = it + 1 < NT;
+
+      const T* qs = Stage + buf * L::STAGE_ELEMS;
+      const T* dos = qs + 32 * L::QSTR;
+      const int arow = unperm32(x);
+      frag qA[KS], doA[KS], qT[2], doT[2];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        qA[s] = ld8<T>(qs + arow * L::QSTR + 16 * g + 8 * s);
+        doA[s] = ld8<T>(dos + arow * L::QSTR + 16 * g + 8 * s);
+      }
+      const frag qaugA = make_aug<T>(ones_g, g == 0 ? Lpk[buf * 32 + arow] : 0u);
+      const frag doaugA = make_aug<T>(g == 0 ? Dpk[buf * 32 + arow] : 0u, 0u);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        doT[u] = TrRead<T>::read(dos, L::QSTR, 8 * u + 8 * g, g, l, dsel_chunk<DP>(0, l), dsel<DP>(0, x));
+        qT[u] = TrRead<T>::read(qs, L::QSTR, 8 * u + 8 * g, g, l, dsel_chunk<DP>(0, l), dsel<DP>(0, x));
+      }
+      f32x16 z = mma(qaugA, maugB, bzn);
+      // Everything for the next step is requested here, AFTER the last use of the bias registers: the
+      // vector-memory counter retires in order, so a wait for older loads never covers these.  The
+      // last step repeats its own loads rather than branching around them.
+      __builtin_amdgcn_sched_barrier(0);
+      load_bias(more ? it + 1 : it);
+      fetch_q(more ? it + 1 : it);
+      __builtin_amdgcn_sched_barrier(0);
+      if (it > 0) reduce_dq(it - 1);
+      fetch_dq_old(it);
+      f32x16 dp = mma(doaugA, vaugB, acc_zero());
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        z = mma(qA[s], kf[s], z);
+        dp = mma(doA[s], vf[s], dp);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pr = fast_exp2(z[i] * cexp);
+        z[i] = pr;
+        dp[i] = pr * dp[i];
+      }
+      frag pf[2], dsf[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) { pf[u] = acc_half<T>(z, u); dsf[u] = acc_half<T>(dp, u); }
+      // dS, rows = keys, through this wavefront's LDS tile and back transposed.  LDS operations of one
+      // wavefront execute in program order, which is all the ordering this exchange needs; the dV / dK
+      // products run while it is in flight.
+      st8<T>(Trw + x * L::TSTR + 16 * g, dsf[0]);
+      st8<T>(Trw + x * L::TSTR + 16 * g + 8, dsf[1]);
+      frag dsT[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) dsT[u] = TrRead<T>::read(Trw, L::TSTR, 8 * u + 8 * g, g, l, plain_chunk(l), x);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        dv = mma(doT[u], pf[u], dv);
+        dk = mma(qT[u], dsf[u], dk);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      f32x16 dq = mma(kT[0], dsT[0], acc_zero());
+      dq = mma(kT[1], dsT[1], dq);
+
+      // partial dQ^T -> this step's slab: lane (x = query, g) owns 16 contiguous columns
+      float* slab = Slw + buf * (32 * L::SSTR);
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        f32x4 v;
+        v[0] = dq[4 * c4]; v[1] = dq[4 * c4 + 1]; v[2] = dq[4 * c4 + 2]; v[3] = dq[4 * c4 + 3];
+        *reinterpret_cast<f32x4*>(slab + x * L::SSTR + 16 * g + 4 * c4) = v;
+      }
+      if (more) stash_q(it + 1, buf ^ 1, kc == 0);
+      barrier_keep_vm<63>();   // LDS hand-over only: global loads / stores stay in flight
+
+    }
+    reduce_dq(NT - 1);
+
+    if (j < S) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int d0 = 16 * g + 8 * u;
+        if (d0 < D) {
+          f32x16 dks = dk;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) dks[i] *= p.scale;
+          st8<T>(dKg + (int64_t)j * p.dk.ss + d0, acc_half<T>(dks, u));
+          st8<T>(dVg + (int64_t)j * p.dv.ss + d0, acc_half<T>(dv, u));
+        }
+      }
+    }
+    __syncthreads();   // the next chunk restages K and the first query tile
+  }
+}
+
+template <typename T, int MAXT, int MINW>
+static hipError_t launch_dqkv_rk_t(const EvoParams& p, int NW, hipStream_t stream) {
+  const size_t smem = RkLayout<T>::smem(NW);
+  if (smem > 160 * 1024) return hipErrorInvalidValue;
+  const long long blocks = (long long)round_up(p.B * p.N, 8) * p.H;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  auto kern = evo_bwd_dqkv_rk_kernel<T, MAXT, MINW>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * NW), smem, stream, p);
+  return hipGetLastError();
+}
+
+// Wavefronts per work-group for the register-resident variant.  A compute unit holds 8 of its
+// wavefronts (2 per SIMD), i.e. floor(8 / NW) work-groups; the estimate of the time per (b, n, h) is
+// (key chunks * NW) / (resident wavefronts).  Ties go to fewer chunks.  MF_DQKV_NW overrides.
+template <typename T> static hipError_t launch_dqkv_rk(const EvoParams& p, hipStream_t stream) {
+  const int NT = (p.S + 31) / 32;
+  int best_nw = 4;
+  long long best_cost = -1;
+  for (int nw = 4; nw <= 8; ++nw) {
+    const int chunks = (NT + nw - 1) / nw;
+    const int resident = nw * (8 / nw);
+    const long long cost = ((long long)chunks * nw * 840 / resident) * 64 + chunks;
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_nw = nw; }
+  }
+  if (const char* e = getenv("MF_DQKV_NW")) { const int v = atoi(e); if (v >= 4 && v <= 8) best_nw = v; }
+  if (best_nw == 4) return launch_dqkv_rk_t<T, 256, 2>(p, 4, stream);
+  return launch_dqkv_rk_t<T, 512, 1>(p, best_nw, stream);
+}
+
 template <typename T, int DP, int TPW> static size_t dqkv_smem(int NW) {
   using L = BwdLayout<T, DP>;
-  return (size_t)NW * TPW * 32 * L::KSTR * sizeof(T) + (size_t)2 * L::STAGE_ELEMS * sizeof(T) + 128 * 4 +
-         (size_t)NW * L::WAVE_BYTES;
+  return (size_t)NW * TPW * 32 * L::QSTR * sizeof(T) + (size_t)2 * L::STAGE_ELEMS * sizeof(T) + 128 * 4 +
+         (size_t)NW * L::wave_bytes(TPW);
 }
 
 template <typename T, int DP, int TPW, int MAXT>
@@ -368,41 +685,32 @@ static hipError_t launch_dqkv_t(const EvoParams& p, int NW, hipStream_t stream) 
   return hipGetLastError();
 }
 
-// Wavefronts per work-group (NW) and key tiles per wavefront (TPW).  Preference order: fewest key
-// chunks (one chunk means dQ is written once, never read back), then fewest idle tile slots, then
-// the larger TPW (more reuse of the staged query tile).  A configuration must fit the 160 KiB LDS.
-// MF_DQKV_NW / MF_DQKV_TPW override the choice (tuning aid).
+// Wavefronts per work-group (NW) of the general kernel, one key tile per wavefront.  Preference order:
+// fewest key chunks (one chunk means dQ is written once, never read back), then fewest idle tile
+// slots, then the smaller group.  fp32 with D > 32 needs more than 256 registers per lane and runs
+// with four wavefronts (one per SIMD).  MF_DQKV_NW overrides the choice (tuning aid).
 template <typename T, int DP> static hipError_t launch_dqkv_d(const EvoParams& p, hipStream_t stream) {
   const int NT = (p.S + 31) / 32;
-  constexpr int max_tpw = (sizeof(T) == 4 || DP > 32) ? 1 : 3;
-  int best_nw = 4, best_tpw = 1;
+  constexpr bool kWide = sizeof(T) == 4 && DP > 32;
+  const int max_nw = kWide ? 4 : 8;
+  int best_nw = 4;
   long long best_cost = -1;
-  for (int tpw = 1; tpw <= max_tpw; ++tpw) {
-    const int max_nw = tpw == 1 ? 16 : 8;
-    for (int nw = 4; nw <= max_nw; ++nw) {
-      const size_t smem = tpw == 1 ? dqkv_smem<T, DP, 1>(nw) : tpw == 2 ? dqkv_smem<T, DP, 2>(nw) : dqkv_smem<T, DP, 3>(nw);
-      if (tpw > max_tpw) continue;
-      if (smem > 160 * 1024) continue;
-      const int slots = nw * tpw;
-      const int chunks = (NT + slots - 1) / slots;
-      const long long cost = ((long long)chunks << 40) + ((long long)(chunks * slots - NT) << 20) + (16 - tpw) * 32 + nw;
-      if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_nw = nw; best_tpw = tpw; }
-    }
+  for (int nw = 4; nw <= max_nw; ++nw) {
+    if (dqkv_smem<T, DP, 1>(nw) > 160 * 1024) continue;
+    const int chunks = (NT + nw - 1) / nw;
+    const long long cost = ((long long)chunks << 40) + ((long long)(chunks * nw - NT) << 20) + nw;
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_nw = nw; }
   }
   if (best_cost < 0) return hipErrorInvalidValue;
-  if (const char* e = getenv("MF_DQKV_TPW")) { const int v = atoi(e); if (v >= 1 && v <= max_tpw) best_tpw = v; }
-  if (const char* e = getenv("MF_DQKV_NW")) { const int v = atoi(e); if (v >= 4 && v <= (best_tpw == 1 ? 16 : 8)) best_nw = v; }
-  if (best_tpw == 1) {
-    return best_nw <= 8 ? launch_dqkv_t<T, DP, 1, 512>(p, best_nw, stream) : launch_dqkv_t<T, DP, 1, 1024>(p, best_nw, stream);
-  }
-  if constexpr (max_tpw >= 3) {
-    if (best_tpw == 2) return launch_dqkv_t<T, DP, 2, 512>(p, best_nw, stream);
-    return launch_dqkv_t<T, DP, 3, 512>(p, best_nw, stream);
-  }
-  return hipErrorInvalidValue;
+  if (const char* e = getenv("MF_DQKV_NW")) { const int v = atoi(e); if (v >= 4 && v <= max_nw) best_nw = v; }
+  if constexpr (kWide) return launch_dqkv_t<T, DP, 1, 256>(p, 4, stream);
+  else return launch_dqkv_t<T, DP, 1, 512>(p, best_nw, stream);
 }
 
 template <typename T> static hipError_t launch_dqkv_s(const EvoParams& p, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (p.D <= 32) return launch_dqkv_rk<T>(p, stream);
+  }
   if (p.D <= 32) return launch_dqkv_d<T, 32>(p, stream);
   if (p.D <= 64) return launch_dqkv_d<T, 64>(p, stream);
   return hipErrorInvalidValue;
@@ -476,42 +784,45 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
   frag qaug = frag_zero<T>();
   if (g == 0) { qaug[0] = (T)1.0f; qaug[1] = (T)1.0f; }
 
+  // Staging registers.  fetch() only ISSUES loads (clamped addresses, no arithmetic on the results), so
+  // that no wait for them lands before the place that consumes them one row later; zeroing of padded
+  // columns / rows and every conversion happens there.
   frag kreg[PF], vreg[PF];
-  float mreg = 0.0f;
+  unsigned mraw = 0u;
   frag qf[KS], dof[KS];
-  float l2 = 0.0f, dl = 0.0f;
+  float lraw = 0.0f, draw = 0.0f;
+  const int mask_es = p.mask_dtype == MF_F32 ? 4 : (p.mask_dtype == MF_F16 || p.mask_dtype == MF_BF16) ? 2 : 1;
+  const int mj = jt0 * 32 + tid < S ? jt0 * 32 + tid : S - 1;     // mask column of the threads tid < ROWS
   auto fetch = [&](int n) {
     const T* kn = Kg + (int64_t)n * p.k.sn;
     const T* vn = Vg + (int64_t)n * p.v.sn;
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int c = tid + 256 * i;
-      kreg[i] = frag_zero<T>(); vreg[i] = frag_zero<T>();
-      if (c < ITEMS) {
-        const int kk = c / CPR, dc = c % CPR;
-        const int j = jt0 * 32 + kk;
-        if (j < S && 8 * dc < D) {
-          kreg[i] = ld8<T>(kn + (int64_t)j * p.k.ss + 8 * dc);
-          vreg[i] = ld8<T>(vn + (int64_t)j * p.v.ss + 8 * dc);
-        }
-      }
+      const int kk = (c < ITEMS ? c : 0) / CPR, dc = c % CPR;
+      int j = jt0 * 32 + kk;
+      j = j < S ? j : S - 1;
+      const int d0 = 8 * dc < D ? 8 * dc : 0;
+      kreg[i] = ld8<T>(kn + (int64_t)j * p.k.ss + d0);
+      vreg[i] = ld8<T>(vn + (int64_t)j * p.v.ss + d0);
     }
-    if (tid < ROWS) {
-      const int j = jt0 * 32 + tid;
-      mreg = j < S ? load_any(p.mask, p.mask_dtype, b * p.mask_sb + n * p.mask_sn + (int64_t)j * p.mask_sj) * inv_scale
-                   : -__builtin_inff();
+    {
+      const unsigned char* mp = reinterpret_cast<const unsigned char*>(p.mask) +
+                                (b * p.mask_sb + n * p.mask_sn + (int64_t)mj * p.mask_sj) * mask_es;
+      if (mask_es == 4) mraw = *reinterpret_cast<const unsigned*>(mp);
+      else if (mask_es == 2) mraw = *reinterpret_cast<const unsigned short*>(mp);
+      else mraw = *mp;
     }
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d0 = (DP / 2) * g + 8 * s;
-      const bool ok = qi < S && d0 < D;
-      qf[s] = ok ? ld8<T>(Qg + (int64_t)n * p.q.sn + d0) : frag_zero<T>();
-      dof[s] = ok ? ld8<T>(dOg + (int64_t)n * p.dO.sn + d0) : frag_zero<T>();
+      const int dcl = d0 < D ? d0 : 0;
+      qf[s] = ld8<T>(Qg + (int64_t)n * p.q.sn + dcl);
+      dof[s] = ld8<T>(dOg + (int64_t)n * p.dO.sn + dcl);
     }
     const int64_t ridx = (((int64_t)b * p.N + n) * p.H + h) * S + qi_c;
-    const float lse = p.lse[ridx];
-    l2 = (qi < S && lse != -__builtin_inff()) ? lse * MF_LOG2E : __builtin_inff();
-    dl = p.delta[ridx];
+    lraw = p.lse[ridx];
+    draw = p.delta[ridx];
   };
   auto stash = [&](int buf) {
     T* kd = Ks + buf * ROWS * L::KSTR;
@@ -522,15 +833,22 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
       if (c < ITEMS) {
         const int kk = c / CPR, dc = c % CPR;
         const int row = (kk & ~31) + perm32(kk & 31);
-        st8<T>(kd + row * L::KSTR + 8 * dc, kreg[i]);
-        st8<T>(vd + row * L::QSTR + 8 * dc, vreg[i]);
+        const bool ok = jt0 * 32 + kk < S && 8 * dc < D;
+        st8<T>(kd + row * L::KSTR + 8 * dc, ok ? kreg[i] : frag_zero<T>());
+        st8<T>(vd + row * L::QSTR + 8 * dc, ok ? vreg[i] : frag_zero<T>());
       }
     }
     if (tid < ROWS) {
+      float mv;
+      if (mask_es == 4) mv = __builtin_bit_cast(float, mraw);
+      else if (p.mask_dtype == MF_F16) mv = (float)__builtin_bit_cast(f16_t, (unsigned short)mraw);
+      else if (p.mask_dtype == MF_BF16) mv = __builtin_bit_cast(float, mraw << 16);
+      else mv = mraw ? 0.0f : -__builtin_inff();
+      mv = jt0 * 32 + tid < S ? mv * inv_scale : -__builtin_inff();
       const int row = (tid & ~31) + perm32(tid & 31);
       frag a = frag_zero<T>();
       T hi, lo;
-      split_hi_lo<T>(mreg, hi, lo);
+      split_hi_lo<T>(mv, hi, lo);
       a[0] = hi; a[1] = lo;
       st8<T>(kd + row * L::KSTR + DP, a);
       st8<T>(kd + row * L::KSTR + DP + 8, frag_zero<T>());
@@ -544,11 +862,20 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
       // operands of this row move from the staging registers to their working copies
       frag qc[KS], doc[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) { qc[s] = qf[s]; doc[s] = dof[s]; }
-      const float l2c = l2, dlc = dl;
+      for (int s = 0; s < KS; ++s) {
+        const bool ok = qi < S && (DP / 2) * g + 8 * s < D;
+        qc[s] = ok ? qf[s] : frag_zero<T>();
+        doc[s] = ok ? dof[s] : frag_zero<T>();
+      }
+      const float l2c = (qi < S && lraw != -__builtin_inff()) ? lraw * MF_LOG2E : __builtin_inff();
+      float dlc = draw;
+      float l2p = l2c;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) { pin(qc[s]); pin(doc[s]); }
+      pin(l2p); pin(dlc);
       stash(buf);
       __syncthreads();
-      if (n + 1 < n_end) fetch(n + 1);
+      fetch(n + 1 < n_end ? n + 1 : n);   // the last row is fetched twice rather than branching around loads
 
       const T* kt = Ks + buf * ROWS * L::KSTR;
       const T* vt = Vs + buf * ROWS * L::QSTR;
@@ -566,7 +893,7 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2c));
+            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2p));
             acc[t][r] = __builtin_fmaf(pr, dp[r] - dlc, acc[t][r]);
           }
         }

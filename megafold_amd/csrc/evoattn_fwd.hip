@@ -277,6 +277,11 @@ __global__ void __launch_bounds__(256, WPE) evo_fwd_kernel(const EvoParams p, co
     }
 
     if (more) stash(buf ^ 1);
+    // Everything requested at the top of this stage (the next tile's K/V and bias) is a whole stage old
+    // here.  Draining it explicitly tells the compiler that nothing is in flight at the loop head;
+    // without that it makes the first use of the bias registers wait for ALL outstanding loads,
+    // including the ones the next stage has only just issued.
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), other counters untouched
     __syncthreads();
   };
 
@@ -284,6 +289,7 @@ __global__ void __launch_bounds__(256, WPE) evo_fwd_kernel(const EvoParams p, co
   fetch(0);
   load_bias(0, bzA);
   stash(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): see the end of stage()
   __syncthreads();
 
   for (int jt = 0; jt < NT; jt += 2) {
