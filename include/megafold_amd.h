@@ -60,11 +60,14 @@ const char* mf_last_error(void);
  * 16 bytes; pointers 16-byte aligned.
  * A query row whose keys are all masked with -inf yields o = 0, lse = -inf and zero gradients.
  * ---------------------------------------------------------------------------------------------- */
-/* Backward phases.  MF_EVO_BWD_DQKV writes dq, dk, dv and leaves rowsum(dO * o) in the workspace;
- * MF_EVO_BWD_DBIAS reads it and writes dbias, so it must follow a DQKV call on the same stream with
- * the same workspace.  phases = 0 runs both (the second only when dbias != NULL). */
+/* Backward phases.  MF_EVO_BWD_PREP copies the pair bias into the workspace (scaled, padded, fp32);
+ * MF_EVO_BWD_DQKV needs that copy, writes dq, dk, dv and leaves rowsum(dO * o) in the workspace;
+ * MF_EVO_BWD_DBIAS needs both and writes dbias.  A call with a subset of the phases must therefore
+ * follow calls for the earlier ones on the same stream with the same workspace.  phases = 0 runs
+ * all of them (DBIAS only when dbias != NULL). */
 #define MF_EVO_BWD_DQKV 1
 #define MF_EVO_BWD_DBIAS 2
+#define MF_EVO_BWD_PREP 4
 
 typedef struct mf_evoattn_args {
   int32_t B, N, S, H, D;

@@ -80,7 +80,7 @@ EvoTensor tens(const void* p, const int64_t* st) {
   return EvoTensor{const_cast<void*>(p), st[0], st[1], st[2], st[3]};
 }
 
-int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStream_t stream) {
+int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStream_t stream, bool prep) {
   p = EvoParams{};
   p.B = a->B; p.N = a->N; p.S = a->S; p.H = a->H; p.D = a->D;
   p.dtype = a->dtype;
@@ -93,10 +93,12 @@ int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStrea
   unsigned char* ws = static_cast<unsigned char*>(a->workspace);
   float* b32 = reinterpret_cast<float*>(ws + pl.off_bias);
   if (a->scale <= 0.0f) return fail(MF_ERR_SHAPE, "scale must be positive (got %g)", (double)a->scale);
-  hipError_t e = launch_bias_prep(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
-                                  a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_rows, pl.bias_ld, 1.0f / a->scale,
-                                  stream);
-  if (e != hipSuccess) return (int)e;
+  if (prep) {
+    hipError_t e = launch_bias_prep(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
+                                    a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_rows, pl.bias_ld,
+                                    1.0f / a->scale, stream);
+    if (e != hipSuccess) return (int)e;
+  }
   p.bias = b32;
   p.bias_sb = (int64_t)a->H * pl.bias_rows * pl.bias_ld;
   p.bias_sh = (int64_t)pl.bias_rows * pl.bias_ld;
@@ -128,7 +130,7 @@ extern "C" int mf_evoattn_fwd(const mf_evoattn_args* a) {
   if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   EvoParams p;
-  rc = fill_params(a, pl, p, stream);
+  rc = fill_params(a, pl, p, stream, true);
   if (rc) return rc;
   return (int)launch_evo_fwd(p, stream);
 }
@@ -142,15 +144,16 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   if ((rc = check_tensor("dk", a->dk, a->dk_stride, es))) return rc;
   if ((rc = check_tensor("dv", a->dv, a->dv_stride, es))) return rc;
   if (a->dbias && !aligned16(a->dbias)) return fail(MF_ERR_ALIGN, "dbias is not 16-byte aligned");
-  if (a->phases < 0 || a->phases > (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS)) return fail(MF_ERR_SHAPE, "phases %d unknown", a->phases);
+  if (a->phases < 0 || a->phases > (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS | MF_EVO_BWD_PREP)) return fail(MF_ERR_SHAPE, "phases %d unknown", a->phases);
   const Plan pl = make_plan(a, true);
   if (!a->workspace || a->workspace_bytes < pl.total)
     return fail(MF_ERR_WORKSPACE, "backward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
                 (unsigned long long)(a->workspace ? a->workspace_bytes : 0));
   if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const int phases = a->phases == 0 ? (MF_EVO_BWD_PREP | MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;
   EvoParams p;
-  rc = fill_params(a, pl, p, stream);
+  rc = fill_params(a, pl, p, stream, (phases & MF_EVO_BWD_PREP) != 0);
   if (rc) return rc;
   unsigned char* ws = static_cast<unsigned char*>(a->workspace);
   p.dO = tens(a->dO, a->do_stride);
@@ -164,7 +167,6 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
 #endif
   p.rows_per_chunk = pl.rows_per_chunk;
   p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
-  const int phases = a->phases == 0 ? (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;
   hipError_t e = hipSuccess;
   if (phases & MF_EVO_BWD_DQKV) {
     e = launch_evo_bwd_dqkv(p, stream);

@@ -120,9 +120,9 @@ def evoattention_forward(Q, K, V, res_mask, pair_bias):
 def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None):
     """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state.
 
-    ``phase_hook(name)``, if given, is called before and after each of the two backward phases
-    ("dqkv", "dbias"), which are then enqueued by two separate C-ABI calls (used by the benchmark to
-    bracket each kernel with events on the launch stream)."""
+    ``phase_hook(name)``, if given, is called before and after each backward phase ("prep", "dqkv",
+    "dbias"), which are then enqueued by separate C-ABI calls (used by the benchmark to bracket each
+    kernel with events on the launch stream)."""
     B, N, S, H, D = Q.shape
     if dO.dtype != Q.dtype:
         dO = dO.to(Q.dtype)
@@ -148,7 +148,8 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phas
         if phase_hook is None:
             _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd")
         else:
-            for name, bit in (("dqkv", _lib.MF_EVO_BWD_DQKV), ("dbias", _lib.MF_EVO_BWD_DBIAS)):
+            for name, bit in (("prep", _lib.MF_EVO_BWD_PREP), ("dqkv", _lib.MF_EVO_BWD_DQKV),
+                              ("dbias", _lib.MF_EVO_BWD_DBIAS)):
                 if bit == _lib.MF_EVO_BWD_DBIAS and dbias is None:
                     continue
                 a.phases = bit
