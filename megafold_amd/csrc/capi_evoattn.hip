@@ -13,18 +13,17 @@ using namespace mf;
 namespace {
 
 struct Plan {
-  int bias_rows, bias_ld;   // padded shape of the fp32 bias/scale copy the kernels read
+  int bias_nt;              // 32 x 32 tiles per side of the fp32 bias/scale copy the kernels read
   uint64_t off_bias, off_delta, off_part, total;
   int n_chunks, rows_per_chunk;
 };
 
 Plan make_plan(const mf_evoattn_args* a, bool backward) {
   Plan pl{};
-  pl.bias_rows = round_up(a->S, 32);
-  pl.bias_ld = round_up(a->S, 64);
+  pl.bias_nt = (a->S + 31) / 32;
   uint64_t off = 0;
   pl.off_bias = off;
-  off += align256((uint64_t)a->B * a->H * pl.bias_rows * pl.bias_ld * 4);
+  off += align256((uint64_t)a->B * a->H * pl.bias_nt * pl.bias_nt * 4096);
   pl.n_chunks = 1;
   pl.rows_per_chunk = a->N;
   if (backward) {
@@ -80,7 +79,7 @@ EvoTensor tens(const void* p, const int64_t* st) {
   return EvoTensor{const_cast<void*>(p), st[0], st[1], st[2], st[3]};
 }
 
-int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStream_t stream, bool prep) {
+int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStream_t stream, bool prep, bool backward) {
   p = EvoParams{};
   p.B = a->B; p.N = a->N; p.S = a->S; p.H = a->H; p.D = a->D;
   p.dtype = a->dtype;
@@ -95,14 +94,13 @@ int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStrea
   if (a->scale <= 0.0f) return fail(MF_ERR_SHAPE, "scale must be positive (got %g)", (double)a->scale);
   if (prep) {
     hipError_t e = launch_bias_prep(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
-                                    a->bias_stride[3], b32, a->B, a->H, a->S, pl.bias_rows, pl.bias_ld,
-                                    1.0f / a->scale, stream);
+                                    a->bias_stride[3], b32, a->B, a->H, a->S, 1.0f / a->scale, backward, stream);
     if (e != hipSuccess) return (int)e;
   }
   p.bias = b32;
-  p.bias_sb = (int64_t)a->H * pl.bias_rows * pl.bias_ld;
-  p.bias_sh = (int64_t)pl.bias_rows * pl.bias_ld;
-  p.bias_ld = pl.bias_ld;
+  p.bias_sb = (int64_t)a->H * pl.bias_nt * pl.bias_nt * 1024;
+  p.bias_sh = (int64_t)pl.bias_nt * pl.bias_nt * 1024;
+  p.bias_nt = pl.bias_nt;
   return 0;
 }
 
@@ -130,7 +128,7 @@ extern "C" int mf_evoattn_fwd(const mf_evoattn_args* a) {
   if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   EvoParams p;
-  rc = fill_params(a, pl, p, stream, true);
+  rc = fill_params(a, pl, p, stream, true, false);
   if (rc) return rc;
   return (int)launch_evo_fwd(p, stream);
 }
@@ -153,7 +151,7 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   const int phases = a->phases == 0 ? (MF_EVO_BWD_PREP | MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;
   EvoParams p;
-  rc = fill_params(a, pl, p, stream, (phases & MF_EVO_BWD_PREP) != 0);
+  rc = fill_params(a, pl, p, stream, (phases & MF_EVO_BWD_PREP) != 0, true);
   if (rc) return rc;
   unsigned char* ws = static_cast<unsigned char*>(a->workspace);
   p.dO = tens(a->dO, a->do_stride);

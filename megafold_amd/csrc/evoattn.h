@@ -19,12 +19,18 @@ struct EvoParams {
   int dtype;       // MF_F32 / MF_F16 / MF_BF16: element type of q, k, v, o, dO, dq, dk, dv
   float scale;     // softmax scale, D^-0.5 in the reference (evoattention.py:705)
   EvoTensor q, k, v, o;
-  // Pair bias DIVIDED BY scale as fp32 [B, H, Sr, bias_ld] with Sr = round_up(S, 32) rows and
-  // bias_ld = round_up(S, 64) columns, zero padded (built in the workspace by launch_bias_prep), so
-  // the kernels read it without bounds checks; row (b, h, i) starts at
-  // bias + b*bias_sb + h*bias_sh + i*bias_ld.
+  // Pair bias DIVIDED BY scale, fp32, zero padded to whole 32 x 32 tiles and stored tile by tile in the
+  // order the consuming lanes hold it (built in the workspace by launch_bias_prep), so that a tile is
+  // four perfectly coalesced 1 KiB loads and can be used directly as the C operand of the score MFMA.
+  // With nt = ceil(S / 32), l = 32 g + x the lane and c4 = 0..3 the load:
+  //   forward layout   tile (qt, jt) at ((qt nt + jt) 1024), float4 (c4 64 + l) =
+  //                    bias[32 qt + x][32 jt + 16 g + 4 c4 + 0..3]          (lane = query, registers = keys)
+  //   backward layout  tile (jt, it) at ((jt nt + it) 1024), float4 (c4 64 + l) =
+  //                    bias[32 it + 16 g + 4 c4 + 0..3][32 jt + x]          (lane = key, registers = queries)
+  // bias_sb / bias_sh are the element strides of the batch and head dimensions.
   const float* bias;
-  int64_t bias_sb, bias_sh, bias_ld;
+  int64_t bias_sb, bias_sh;
+  int bias_nt;
   // Additive key mask [B, N, S] in its own dtype (MF_BOOL: keep-mask, true -> 0, false -> -inf).
   const void* mask;
   int mask_dtype;
@@ -47,9 +53,10 @@ struct EvoParams {
 hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dbias(const EvoParams& p, hipStream_t stream);
-// bias (any float dtype, any strides) * mult -> fp32 [B, H, Sr, ld], zero padded for i >= S or j >= S.
+// bias (any float dtype, any strides) * mult -> the tiled fp32 copy described at EvoParams::bias;
+// `backward_layout` selects which of the two orders is written.
 hipError_t launch_bias_prep(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
-                            int B, int H, int S, int Sr, int ld, float mult, hipStream_t stream);
+                            int B, int H, int S, float mult, bool backward_layout, hipStream_t stream);
 
 // Number of rows of N one work-group of the bias-gradient kernel walks over, chosen so the grid
 // fills the device while the partial-sum workspace stays small.

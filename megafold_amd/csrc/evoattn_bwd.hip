@@ -176,8 +176,9 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
       const float mv = j < S ? load_any(p.mask, p.mask_dtype, mask_base + (int64_t)j * p.mask_sj) * inv_scale
                              : -__builtin_inff();
       mk[t] = g == 0 ? pack_split<T>(mv) : 0u;
-      // bias/scale copy is zero padded to whole tiles: register i of half g <-> query 32*it + 16*g + i
-      bias_t[t] = biasg + (int64_t)(16 * g) * p.bias_ld + (tile_ok[t] ? j0 : 0) + x;
+      // column of bias tiles of this key tile (backward layout, see EvoParams::bias): register i of half g
+      // <-> query 32*it + 16*g + i
+      bias_t[t] = biasg + (int64_t)(tile_ok[t] ? j0 >> 5 : 0) * p.bias_nt * 1024 + 4 * l;
     }
     f32x16 dk[TPW][DT], dv[TPW][DT];
 #pragma unroll
@@ -188,9 +189,12 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
     // bias/scale tile of the next (query tile, key tile) step, loaded one step ahead
     f32x16 bzn;
     auto load_bias = [&](int it, const float* base) {
-      const float* bp = base + (int64_t)it * 32 * p.bias_ld;
+      const float* bp = base + it * 1024;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) bzn[i] = bp[i * (int)p.bias_ld];
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(bp + 256 * c4);
+        bzn[4 * c4] = v[0]; bzn[4 * c4 + 1] = v[1]; bzn[4 * c4 + 2] = v[2]; bzn[4 * c4 + 3] = v[3];
+      }
     };
     load_bias(0, bias_t[0]);   // idle tile slots read (and ignore) column block 0
 
@@ -474,12 +478,15 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
                            : -__builtin_inff();
     const frag maugB = make_aug<T>(g == 0 ? pack_split<T>(mv) : 0u, ones_g);
     // bias/scale copy is zero padded to whole tiles: register i of half g <-> query 32*it + 16*g + i
-    const float* bias_t = biasg + (int64_t)(16 * g) * p.bias_ld + (j0 < S ? j0 : 0) + x;
+    const float* bias_t = biasg + (int64_t)(j0 < S ? j0 >> 5 : 0) * p.bias_nt * 1024 + 4 * l;
     f32x16 bzn;
     auto load_bias = [&](int it) {
-      const float* bp = bias_t + (int64_t)it * 32 * p.bias_ld;
+      const float* bp = bias_t + it * 1024;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) bzn[i] = bp[i * (int)p.bias_ld];
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(bp + 256 * c4);
+        bzn[4 * c4] = v[0]; bzn[4 * c4 + 1] = v[1]; bzn[4 * c4 + 2] = v[2]; bzn[4 * c4 + 3] = v[3];
+      }
     };
     load_bias(0);
 
@@ -778,7 +785,11 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int j = (jt0 + t) * 32 + 16 * g + r;
-      bz[t][r] = j < p.bias_ld ? biasg[(int64_t)qi_c * p.bias_ld + j] : 0.0f;
+      // element (query qi, key j) of the backward-layout tile (j / 32, qi / 32)
+      const int qq = qi_c & 31;
+      bz[t][r] = j < 32 * p.bias_nt
+                     ? biasg[((int64_t)(j >> 5) * p.bias_nt + (qi_c >> 5)) * 1024 + (((qq & 15) >> 2) * 64 + 32 * (qq >> 4) + (j & 31)) * 4 + (qq & 3)]
+                     : 0.0f;
     }
   }
   frag qaug = frag_zero<T>();
@@ -905,12 +916,21 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
   float* dst = (p.n_chunks > 1 ? p.dbias_part + (int64_t)chunk * p.B * p.H * S * S : p.dbias) +
                ((int64_t)b * p.H + h) * S * S;
   if (qi < S) {
+    const bool vec = (S & 3) == 0;     // rows of the gradient are 16-byte aligned
 #pragma unroll
     for (int t = 0; t < TR; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int j = (jt0 + t) * 32 + 16 * g + r;
-        if (j < S) dst[(int64_t)qi * S + j] = acc[t][r];
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const int j = (jt0 + t) * 32 + 16 * g + 4 * c4;
+        float* d4 = dst + (int64_t)qi * S + j;
+        if (vec && j + 3 < S) {
+          f32x4 v = {acc[t][4 * c4], acc[t][4 * c4 + 1], acc[t][4 * c4 + 2], acc[t][4 * c4 + 3]};
+          *reinterpret_cast<f32x4*>(d4) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (j + e < S) d4[e] = acc[t][4 * c4 + e];
+        }
       }
   }
 }

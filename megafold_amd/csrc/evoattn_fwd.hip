@@ -135,7 +135,10 @@ __global__ void __launch_bounds__(256, WPE) evo_fwd_kernel(const EvoParams p, co
   const int mask_step = g == 0 ? 32 : 0;
 
   // bias/scale rows are zero padded to whole tiles: no bounds checks on the loads
-  const float* biasp = p.bias + b * p.bias_sb + h * p.bias_sh + (int64_t)qrow_c * p.bias_ld + 16 * g;
+  // this wavefront's row of bias tiles (forward layout, see EvoParams::bias); query tiles past S are
+  // clamped, their rows are never stored
+  const int qt = qb * 4 + w < p.bias_nt ? qb * 4 + w : p.bias_nt - 1;
+  const float* biasp = p.bias + b * p.bias_sb + h * p.bias_sh + (int64_t)qt * p.bias_nt * 1024 + 4 * l;
 
   // ---- staging of one stage.  Source pointers advance by 32 keys per stage; keys past S are
   // clamped to the last key (their logits are -inf through the mask, and P = 0 times a finite V is 0).
@@ -197,10 +200,10 @@ __global__ void __launch_bounds__(256, WPE) evo_fwd_kernel(const EvoParams p, co
   }
 
   auto load_bias = [&](int jt, f32x16& dst) {
-    const float* bp = biasp + jt * 32;
+    const float* bp = biasp + jt * 1024;
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(bp + 4 * c4);
+      const f32x4 v = *reinterpret_cast<const f32x4*>(bp + 256 * c4);
       dst[4 * c4 + 0] = v[0]; dst[4 * c4 + 1] = v[1]; dst[4 * c4 + 2] = v[2]; dst[4 * c4 + 3] = v[3];
     }
   };
@@ -377,29 +380,42 @@ hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream) {
   }
 }
 
-// ---- pair bias of any float dtype / strides -> fp32 [B, H, Sr, ld] times `mult`, zero padded ----------
+// ---- pair bias of any float dtype / strides -> tiled fp32 copy times `mult`, zero padded ------------
+// One thread writes one float4 of the layout described at EvoParams::bias.
 __global__ void __launch_bounds__(256) bias_prep_kernel(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si,
-                                                        int64_t sj, float* dst, int H, int S, int Sr, int ld, float mult,
-                                                        int64_t total) {
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-    const int j = (int)(idx % ld);
-    const int64_t rw = idx / ld;
-    const int i = (int)(rw % Sr);
-    const int64_t bh = rw / Sr;
+                                                        int64_t sj, float* dst, int H, int S, int nt, float mult,
+                                                        int backward_layout, int64_t total4) {
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (int64_t)gridDim.x * 256) {
+    const int l = (int)(idx & 63), c4 = (int)((idx >> 6) & 3);
+    const int64_t tile = idx >> 8;
+    const int t1 = (int)(tile % nt);
+    const int64_t r1 = tile / nt;
+    const int t0 = (int)(r1 % nt);
+    const int64_t bh = r1 / nt;
     const int h = (int)(bh % H);
     const int64_t b = bh / H;
-    dst[idx] = (j < S && i < S) ? load_any(src, dtype, b * sb + h * sh + i * si + j * sj) * mult : 0.0f;
+    const int x = l & 31, g = l >> 5;
+    f32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // forward: tile (qt = t0, jt = t1); backward: tile (jt = t0, it = t1)
+      const int i = backward_layout ? 32 * t1 + 16 * g + 4 * c4 + e : 32 * t0 + x;
+      const int j = backward_layout ? 32 * t0 + x : 32 * t1 + 16 * g + 4 * c4 + e;
+      v[e] = (i < S && j < S) ? load_any(src, dtype, b * sb + h * sh + i * si + j * sj) * mult : 0.0f;
+    }
+    *reinterpret_cast<f32x4*>(dst + 4 * idx) = v;
   }
 }
 
 hipError_t launch_bias_prep(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
-                            int B, int H, int S, int Sr, int ld, float mult, hipStream_t stream) {
-  const int64_t total = (int64_t)B * H * Sr * ld;
-  if (total == 0) return hipSuccess;
-  int64_t blocks = (total + 255) / 256;
+                            int B, int H, int S, float mult, bool backward_layout, hipStream_t stream) {
+  const int nt = (S + 31) / 32;
+  const int64_t total4 = (int64_t)B * H * nt * nt * 256;
+  if (total4 == 0) return hipSuccess;
+  int64_t blocks = (total4 + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   hipLaunchKernelGGL(bias_prep_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dtype, sb, sh, si, sj, dst, H,
-                     S, Sr, ld, mult, total);
+                     S, nt, mult, backward_layout ? 1 : 0, total4);
   return hipGetLastError();
 }
 

@@ -23,6 +23,7 @@
 //        kernel sums the ranges in a fixed order and forms
 //        dW = gamma G + beta s,  dgamma = rowsum(W (.) G),  dbeta = W s,  db = s.
 #pragma once
+#include <cstdlib>
 #include "common.h"
 #include "lnlinear.h"
 
@@ -105,6 +106,8 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
   }
 
   // ---- staging of one block of rows: x -> LDS, statistics on the way ---------------------------
+  // fetch() only issues loads (clamped addresses, nothing touches the results); stash() consumes
+  // them one iteration later, applies the zero padding and forms the row statistics.
   constexpr int items = RB * CPR;
   constexpr int PFMAX = (items + 255) / 256;
   frag xr[PFMAX];
@@ -112,12 +115,10 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
 #pragma unroll
     for (int i = 0; i < PFMAX; ++i) {
       const int item = tid + 256 * i;
-      xr[i] = frag_zero<T>();
-      if (item < items) {
-        const int row = item / CPR, dc = item % CPR;
-        const int64_t m = rb * RB + row;
-        if (m < p.M && 8 * dc < p.K) xr[i] = ld8<T>(X + m * p.K + 8 * dc);
-      }
+      const int row = (item < items ? item : 0) / CPR, dc = item % CPR;
+      int64_t m = rb * RB + row;
+      m = m < p.M ? m : p.M - 1;
+      xr[i] = ld8<T>(X + m * p.K + (8 * dc < p.K ? 8 * dc : 0));
     }
   };
   auto stash = [&](int64_t rb, int buf) {
@@ -127,17 +128,20 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
       const int item = tid + 256 * i;
       if (item < items) {
         const int row = item / CPR, dc = item % CPR;
-        st8<T>(xd + row * L::XSTR + 8 * dc, xr[i]);
+        const int64_t m = rb * RB + row;
+        const bool live = m < p.M && 8 * dc < p.K;
+        const frag xv = live ? xr[i] : frag_zero<T>();
+        st8<T>(xd + row * L::XSTR + 8 * dc, xv);
         float s = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s += to_f(xr[i][e]);
+        for (int e = 0; e < 8; ++e) s += to_f(xv[e]);
 #pragma unroll
         for (int msk = 1; msk < CPR; msk <<= 1) s += __shfl_xor(s, msk);
         const float mu = s / (float)p.K;
         float d = 0.0f;
         if (8 * dc < p.K) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) { const float c = to_f(xr[i][e]) - mu; d += c * c; }
+          for (int e = 0; e < 8; ++e) { const float c = to_f(xv[e]) - mu; d += c * c; }
         }
 #pragma unroll
         for (int msk = 1; msk < CPR; msk <<= 1) d += __shfl_xor(d, msk);
@@ -145,22 +149,26 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
         if (dc == 0) {
           meanL[buf * RB + row] = mu;
           rstdL[buf * RB + row] = rs;
-          const int64_t m = rb * RB + row;
           if (ACT != LN_ACT_SWIGLU_BWD && blockIdx.y == 0 && m < p.M) { p.mean[m] = mu; p.rstd[m] = rs; }
         }
       }
     }
   };
 
+  // Iteration order (G = gridDim.x row blocks apart): the block of this iteration is already in LDS;
+  // after its matrix products the NEXT block's registers (requested one iteration ago, just before
+  // that iteration's output stores) are stashed, the block after that is requested, and only then the
+  // outputs are stored.  The single point that waits for vector memory therefore only ever waits for
+  // loads and stores that are a whole iteration old.
   const int64_t nrb = (p.M + RB - 1) / RB;
+  const int64_t G = gridDim.x;
   int64_t rb = blockIdx.x;
-  if (rb < nrb) fetch(rb);
+  if (rb < nrb) { fetch(rb); stash(rb, 0); }
+  if (rb + G < nrb) fetch(rb + G);
   int it = 0;
-  for (; rb < nrb; rb += gridDim.x, ++it) {
+  for (; rb < nrb; rb += G, ++it) {
     const int buf = it & 1;
-    stash(rb, buf);
     __syncthreads();
-    if (rb + gridDim.x < nrb) fetch(rb + gridDim.x);
 
     const T* xt = Xs + buf * RB * L::XSTR + (wr * 32 + x) * L::XSTR;
     f32x16 acc[NTW];
@@ -172,9 +180,12 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
 #pragma unroll
       for (int t = 0; t < NTW; ++t) acc[t] = mma(af[t][s], bf, acc[t]);
     }
+    const float mu_cur = meanL[buf * RB + wr * 32 + x], rs_cur = rstdL[buf * RB + wr * 32 + x];
+    if (rb + G < nrb) stash(rb + G, buf ^ 1);
+    if (rb + 2 * G < nrb) fetch(rb + 2 * G);
 
     const int64_t m = rb * RB + wr * 32 + x;
-    const float mu = meanL[buf * RB + wr * 32 + x], rs = rstdL[buf * RB + wr * 32 + x];
+    const float mu = mu_cur, rs = rs_cur;
     const float c0 = -rs * mu;
     const float* csw = csL + (wn * NTW) * 32 + 16 * g;
     const float* bpw = bpL + (wn * NTW) * 32 + 16 * g;
@@ -285,7 +296,9 @@ template <typename T, int KP, int ACT> static hipError_t launch_fwd_k(const LnPa
     return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
   } else {
     if (NOUT <= 64) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
-    if (NOUT <= 128 || wide) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
+    // the backward form also holds the incoming gradient and two outputs per column: with four tiles
+    // per wavefront it would spill registers
+    if (NOUT <= 128 || wide || ACT == LN_ACT_SWIGLU_BWD || getenv("MF_LN_NTW2")) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
     return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
   }
 }
