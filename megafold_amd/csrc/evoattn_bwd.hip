@@ -736,7 +736,9 @@ hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream) {
 // dBias
 // =================================================================================================
 template <typename T, int DP, int TR>
-__global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
+__global__ void __launch_bounds__(256, (sizeof(T) == 4 && DP > 32) ? 1 : 2)
+evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
+  constexpr int AHEAD = DP <= 32 ? 2 : 1;
   using L = BwdLayout<T, DP>;
   using frag = frag_t<T>;
   constexpr int KS = DP / 16, CPR = DP / 8;
@@ -795,16 +797,20 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
   frag qaug = frag_zero<T>();
   if (g == 0) { qaug[0] = (T)1.0f; qaug[1] = (T)1.0f; }
 
-  // Staging registers.  fetch() only ISSUES loads (clamped addresses, no arithmetic on the results), so
-  // that no wait for them lands before the place that consumes them one row later; zeroing of padded
-  // columns / rows and every conversion happens there.
-  frag kreg[PF], vreg[PF];
-  unsigned mraw = 0u;
-  frag qf[KS], dof[KS];
-  float lraw = 0.0f, draw = 0.0f;
+  // Staging registers, AHEAD sets: the row consumed in iteration n was requested in iteration
+  // n - AHEAD (two rows of loads in flight where the registers allow it).  fetch() only ISSUES loads (clamped addresses, no
+  // arithmetic on the results); zeroing of padded columns / rows and every conversion happens where
+  // the set is consumed, two iterations later.
+  struct Staged {
+    frag k[PF], v[PF];
+    unsigned mraw;
+    frag q[KS], dO[KS];
+    float lraw, draw;
+  };
+  Staged sA, sB;
   const int mask_es = p.mask_dtype == MF_F32 ? 4 : (p.mask_dtype == MF_F16 || p.mask_dtype == MF_BF16) ? 2 : 1;
   const int mj = jt0 * 32 + tid < S ? jt0 * 32 + tid : S - 1;     // mask column of the threads tid < ROWS
-  auto fetch = [&](int n) {
+  auto fetch = [&](int n, Staged& st) {
     const T* kn = Kg + (int64_t)n * p.k.sn;
     const T* vn = Vg + (int64_t)n * p.v.sn;
 #pragma unroll
@@ -814,28 +820,28 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
       int j = jt0 * 32 + kk;
       j = j < S ? j : S - 1;
       const int d0 = 8 * dc < D ? 8 * dc : 0;
-      kreg[i] = ld8<T>(kn + (int64_t)j * p.k.ss + d0);
-      vreg[i] = ld8<T>(vn + (int64_t)j * p.v.ss + d0);
+      st.k[i] = ld8<T>(kn + (int64_t)j * p.k.ss + d0);
+      st.v[i] = ld8<T>(vn + (int64_t)j * p.v.ss + d0);
     }
     {
       const unsigned char* mp = reinterpret_cast<const unsigned char*>(p.mask) +
                                 (b * p.mask_sb + n * p.mask_sn + (int64_t)mj * p.mask_sj) * mask_es;
-      if (mask_es == 4) mraw = *reinterpret_cast<const unsigned*>(mp);
-      else if (mask_es == 2) mraw = *reinterpret_cast<const unsigned short*>(mp);
-      else mraw = *mp;
+      if (mask_es == 4) st.mraw = *reinterpret_cast<const unsigned*>(mp);
+      else if (mask_es == 2) st.mraw = *reinterpret_cast<const unsigned short*>(mp);
+      else st.mraw = *mp;
     }
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d0 = (DP / 2) * g + 8 * s;
       const int dcl = d0 < D ? d0 : 0;
-      qf[s] = ld8<T>(Qg + (int64_t)n * p.q.sn + dcl);
-      dof[s] = ld8<T>(dOg + (int64_t)n * p.dO.sn + dcl);
+      st.q[s] = ld8<T>(Qg + (int64_t)n * p.q.sn + dcl);
+      st.dO[s] = ld8<T>(dOg + (int64_t)n * p.dO.sn + dcl);
     }
     const int64_t ridx = (((int64_t)b * p.N + n) * p.H + h) * S + qi_c;
-    lraw = p.lse[ridx];
-    draw = p.delta[ridx];
+    st.lraw = p.lse[ridx];
+    st.draw = p.delta[ridx];
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, const Staged& st) {
     T* kd = Ks + buf * ROWS * L::KSTR;
     T* vd = Vs + buf * ROWS * L::QSTR;
 #pragma unroll
@@ -845,16 +851,16 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
         const int kk = c / CPR, dc = c % CPR;
         const int row = (kk & ~31) + perm32(kk & 31);
         const bool ok = jt0 * 32 + kk < S && 8 * dc < D;
-        st8<T>(kd + row * L::KSTR + 8 * dc, ok ? kreg[i] : frag_zero<T>());
-        st8<T>(vd + row * L::QSTR + 8 * dc, ok ? vreg[i] : frag_zero<T>());
+        st8<T>(kd + row * L::KSTR + 8 * dc, ok ? st.k[i] : frag_zero<T>());
+        st8<T>(vd + row * L::QSTR + 8 * dc, ok ? st.v[i] : frag_zero<T>());
       }
     }
     if (tid < ROWS) {
       float mv;
-      if (mask_es == 4) mv = __builtin_bit_cast(float, mraw);
-      else if (p.mask_dtype == MF_F16) mv = (float)__builtin_bit_cast(f16_t, (unsigned short)mraw);
-      else if (p.mask_dtype == MF_BF16) mv = __builtin_bit_cast(float, mraw << 16);
-      else mv = mraw ? 0.0f : -__builtin_inff();
+      if (mask_es == 4) mv = __builtin_bit_cast(float, st.mraw);
+      else if (p.mask_dtype == MF_F16) mv = (float)__builtin_bit_cast(f16_t, (unsigned short)st.mraw);
+      else if (p.mask_dtype == MF_BF16) mv = __builtin_bit_cast(float, st.mraw << 16);
+      else mv = st.mraw ? 0.0f : -__builtin_inff();
       mv = jt0 * 32 + tid < S ? mv * inv_scale : -__builtin_inff();
       const int row = (tid & ~31) + perm32(tid & 31);
       frag a = frag_zero<T>();
@@ -866,49 +872,60 @@ __global__ void __launch_bounds__(256, 2) evo_bwd_dbias_kernel(const EvoParams p
     }
   };
 
-  if (n_begin < n_end) {
-    fetch(n_begin);
-    for (int n = n_begin; n < n_end; ++n) {
-      const int buf = (n - n_begin) & 1;
-      // operands of this row move from the staging registers to their working copies
-      frag qc[KS], doc[KS];
+  // one row n: consume the staged set, publish K / V, request row n + AHEAD into the same set, compute
+  auto row_step = [&](int n, int buf, Staged& st) {
+    frag qc[KS], doc[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const bool ok = qi < S && (DP / 2) * g + 8 * s < D;
-        qc[s] = ok ? qf[s] : frag_zero<T>();
-        doc[s] = ok ? dof[s] : frag_zero<T>();
-      }
-      const float l2c = (qi < S && lraw != -__builtin_inff()) ? lraw * MF_LOG2E : __builtin_inff();
-      float dlc = draw;
-      float l2p = l2c;
+    for (int s = 0; s < KS; ++s) {
+      const bool ok = qi < S && (DP / 2) * g + 8 * s < D;
+      qc[s] = ok ? st.q[s] : frag_zero<T>();
+      doc[s] = ok ? st.dO[s] : frag_zero<T>();
+    }
+    float l2p = (qi < S && st.lraw != -__builtin_inff()) ? st.lraw * MF_LOG2E : __builtin_inff();
+    float dlc = st.draw;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) { pin(qc[s]); pin(doc[s]); }
-      pin(l2p); pin(dlc);
-      stash(buf);
-      __syncthreads();
-      fetch(n + 1 < n_end ? n + 1 : n);   // the last row is fetched twice rather than branching around loads
+    for (int s = 0; s < KS; ++s) { pin(qc[s]); pin(doc[s]); }
+    pin(l2p); pin(dlc);
+    stash(buf, st);
+    __syncthreads();
+    fetch(n + AHEAD < n_end ? n + AHEAD : n_end - 1, st);   // the tail repeats the last row rather than branching around loads
 
-      const T* kt = Ks + buf * ROWS * L::KSTR;
-      const T* vt = Vs + buf * ROWS * L::QSTR;
+    const T* kt = Ks + buf * ROWS * L::KSTR;
+    const T* vt = Vs + buf * ROWS * L::QSTR;
 #pragma unroll
-      for (int t = 0; t < TR; ++t) {
-        if ((jt0 + t) * 32 < S) {
-          const T* krow = kt + (32 * t + x) * L::KSTR;
-          const T* vrow = vt + (32 * t + x) * L::QSTR;
-          f32x16 z = mma(ld8<T>(krow + DP + 8 * g), qaug, bz[t]);
-          f32x16 dp = acc_zero();
+    for (int t = 0; t < TR; ++t) {
+      if ((jt0 + t) * 32 < S) {
+        const T* krow = kt + (32 * t + x) * L::KSTR;
+        const T* vrow = vt + (32 * t + x) * L::QSTR;
+        f32x16 z = mma(ld8<T>(krow + DP + 8 * g), qaug, bz[t]);
+        f32x16 dp = acc_zero();
 #pragma unroll
-          for (int s = 0; s < KS; ++s) {
-            z = mma(ld8<T>(krow + (DP / 2) * g + 8 * s), qc[s], z);
-            dp = mma(ld8<T>(vrow + (DP / 2) * g + 8 * s), doc[s], dp);
-          }
+        for (int s = 0; s < KS; ++s) {
+          z = mma(ld8<T>(krow + (DP / 2) * g + 8 * s), qc[s], z);
+          dp = mma(ld8<T>(vrow + (DP / 2) * g + 8 * s), doc[s], dp);
+        }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2p));
-            acc[t][r] = __builtin_fmaf(pr, dp[r] - dlc, acc[t][r]);
-          }
+        for (int r = 0; r < 16; ++r) {
+          const float pr = fast_exp2(__builtin_fmaf(z[r], cexp, -l2p));
+          acc[t][r] = __builtin_fmaf(pr, dp[r] - dlc, acc[t][r]);
         }
       }
+    }
+  };
+
+  if (n_begin < n_end) {
+    if constexpr (AHEAD == 2) {
+      fetch(n_begin, sA);
+      fetch(n_begin + 1 < n_end ? n_begin + 1 : n_begin, sB);
+      int n = n_begin;
+      for (; n + 1 < n_end; n += 2) {     // both halves unconditional: the loop-carried load order is fixed
+        row_step(n, 0, sA);
+        row_step(n + 1, 1, sB);
+      }
+      if (n < n_end) row_step(n, 0, sA);
+    } else {
+      fetch(n_begin, sA);
+      for (int n = n_begin; n < n_end; ++n) row_step(n, (n - n_begin) & 1, sA);
     }
   }
 
@@ -944,19 +961,42 @@ __global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, fl
 }
 
 // Key tiles per wavefront patch: limited by the registers the patch and its bias seed occupy.
-static int dbias_tr(int dtype, int D) { (void)D; return dtype == MF_F32 ? 1 : 2; }
+static int dbias_tr(int dtype, int D) { return (dtype == MF_F32 || D > 32) ? 1 : 2; }
 
+static int dbias_num_cu() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, n = 0;
+    cached = (hipGetDevice(&dev) == hipSuccess &&
+              hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cached;
+}
+
+// Number of chunks the N rows are split into.  Work-groups of one (b, h, chunk) group are placed on
+// one XCD (they share Q, dO, K, V in its L2) and two work-groups fit a compute unit, so the busiest XCD
+// runs ceil(groups / 8) * regions work-groups in rounds of 2 * CUs / 8, each round lasting
+// ceil(N / chunks) row steps.  Every chunk also costs one partial [B, H, S, S] buffer that is written
+// and read back, priced in row steps (about 1.4 us) at about 2 TB/s so that near-ties go to the
+// smaller workspace.  Pick the chunk count with the smallest estimate.
 int evo_dbias_chunks(int B, int N, int S, int H, int D, int dtype) {
   const int TR = dbias_tr(dtype, D);
   const int NT = (S + 31) / 32;
   const int IB = (S + 127) / 128, JB = (NT + TR - 1) / TR;
-  const long long regions = (long long)B * H * IB * JB;
-  long long want = (768 + regions - 1) / regions;   // ~3 work-groups per compute unit
-  if (want > 8) want = 8;                           // bounds the partial-sum workspace
-  if (want > N) want = N;
-  if (want < 1) want = 1;
-  const int rows = (int)((N + want - 1) / want);
-  return (N + rows - 1) / rows;
+  const long long regions = (long long)IB * JB;
+  const long long slots_xcd = 2LL * (dbias_num_cu() / 8 > 0 ? dbias_num_cu() / 8 : 1);
+  const double part_cost = (double)B * H * S * S * 8.0 / 2.0e12 / 1.4e-6;
+  int best = 1;
+  double best_cost = -1.0;
+  for (int c = 1; c <= 16 && c <= N; ++c) {
+    const int rows = (N + c - 1) / c;
+    if ((N + rows - 1) / rows != c) continue;
+    const long long groups_xcd = ((long long)B * H * c + 7) / 8;
+    const long long rounds = (groups_xcd * regions + slots_xcd - 1) / slots_xcd;
+    const double cost = (double)rounds * rows + (c > 1 ? c * part_cost : 0.0);
+    if (best_cost < 0.0 || cost < best_cost) { best_cost = cost; best = c; }
+  }
+  return best;
 }
 
 template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const EvoParams& p, hipStream_t stream) {
@@ -990,7 +1030,7 @@ template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const Evo
 template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipStream_t stream) {
   constexpr bool wide = sizeof(T) == 4;
   if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 2>(p, stream);
-  if (p.D <= 64) return launch_dbias_t<T, 64, wide ? 1 : 2>(p, stream);
+  if (p.D <= 64) return launch_dbias_t<T, 64, 1>(p, stream);
   return hipErrorInvalidValue;
 }
 

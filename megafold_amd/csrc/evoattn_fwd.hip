@@ -349,12 +349,34 @@ template <typename T, int DP, int R, int WPE> static hipError_t launch_fwd_t(con
   return hipGetLastError();
 }
 
-// Rows per work-group: as many as the register file allows while the grid still fills the device.
+static int fwd_num_cu() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, n = 0;
+    cached = (hipGetDevice(&dev) == hipSuccess &&
+              hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cached;
+}
+
+// Rows n per work-group (R).  More rows share one pair-bias tile, but the grid runs in whole rounds of
+// resident work-groups (3 per compute unit for R = 2, 2 for R = 3 and 4), and a stage costs about
+// 7 + R units of time, so the best R is the one with the smallest rounds * (7 + R) (fitted to
+// measurements at S = 384 and S = 768).  Small problems use fewer rows to keep the device busy.
+// MF_FWD_ROWS overrides.
 template <typename T> static hipError_t launch_fwd_d(const EvoParams& p, hipStream_t stream) {
   constexpr bool wide = sizeof(T) == 4;
+  const long long QB = (p.S + 127) / 128;
   int rows = 4;
+  double best = -1.0;
+  for (int r = 2; r <= 4; ++r) {
+    const long long wgs = (long long)round_up(p.B * ((p.N + r - 1) / r), 8) * p.H * QB;
+    const long long slots = (long long)(r == 2 ? 3 : 2) * fwd_num_cu();
+    const double cost = (double)((wgs + slots - 1) / slots) * (7.0 + r);
+    if (best < 0.0 || cost < best) { best = cost; rows = r; }
+  }
   if (const char* e = getenv("MF_FWD_ROWS")) rows = atoi(e);
-  const long long groups1 = (long long)p.B * p.N * p.H * ((p.S + 127) / 128);
+  const long long groups1 = (long long)p.B * p.N * p.H * QB;
   if (groups1 < 2048) rows = rows > 2 ? 2 : rows;   // small problems: keep enough work-groups
   if (groups1 < 1024 || p.N == 1) rows = 1;
   if constexpr (wide) {
@@ -363,6 +385,7 @@ template <typename T> static hipError_t launch_fwd_d(const EvoParams& p, hipStre
   } else {
     if (p.D <= 32) {
       if (rows >= 4) return launch_fwd_t<T, 32, 4, 2>(p, stream);
+      if (rows == 3) return launch_fwd_t<T, 32, 3, 2>(p, stream);
       if (rows >= 2) return launch_fwd_t<T, 32, 2, 3>(p, stream);
       return launch_fwd_t<T, 32, 1, 4>(p, stream);
     }
