@@ -4,6 +4,7 @@
 // (megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:351-405, 408-474) and swiglu_forward /
 // swiglu_backward (megafold/model/FusedTransition/fused_transition.py:55-93).
 #include "../../include/megafold_amd.h"
+#include <cstdlib>
 #include "capi_common.h"
 #include "common.h"
 #include "lnlinear.h"
@@ -78,6 +79,10 @@ int check(const mf_lnlinear_args* a, bool backward) {
 
 LnParams fill(const mf_lnlinear_args* a, const LnPlan& pl, bool backward) {
   LnParams p{};
+#ifdef MF_TIMELINE
+  { const char* e = getenv("MF_TL_PTR"); p.tl = e ? reinterpret_cast<unsigned*>(strtoull(e, nullptr, 16)) : nullptr;
+    const char* f = getenv("MF_TL_BLOCK"); p.tl_block = f ? atoi(f) : 0; }
+#endif
   p.M = a->M; p.K = a->K; p.N = a->N; p.KP = pl.KP; p.dtype = a->dtype; p.eps = a->eps;
   p.x = a->x; p.gamma = a->gamma; p.beta = a->beta; p.W = a->W; p.b = a->b;
   p.out = a->out; p.mean = a->mean; p.rstd = a->rstd;

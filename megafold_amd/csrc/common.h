@@ -299,6 +299,27 @@ template <> __device__ __forceinline__ unsigned ones_word<float>() { return __bu
 
 }  // namespace mf
 
+// Sum over aligned groups of W consecutive lanes (W = 2, 4, 8, 16 or 32); every lane of a group gets
+// the group's total.  Up to 16 lanes this is pure DPP (quad permutes, then the half-row and row
+// mirrors, which pair up lanes that already hold equal partial sums): no LDS traffic, unlike
+// __shfl_xor, which goes through ds_bpermute and costs an LDS round trip per step.
+template <int W> __device__ __forceinline__ float group_sum(float v) {
+  static_assert(W == 1 || W == 2 || W == 4 || W == 8 || W == 16 || W == 32, "group width");
+  auto dpp_add = [](float a, int ctrl) {
+    const int moved = ctrl == 0xB1   ? __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), 0xB1, 0xF, 0xF, true)
+                      : ctrl == 0x4E ? __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), 0x4E, 0xF, 0xF, true)
+                      : ctrl == 0x141 ? __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), 0x141, 0xF, 0xF, true)
+                                      : __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a), 0x140, 0xF, 0xF, true);
+    return a + __builtin_bit_cast(float, moved);
+  };
+  if (W >= 2) v = dpp_add(v, 0xB1);     // quad_perm [1,0,3,2]
+  if (W >= 4) v = dpp_add(v, 0x4E);     // quad_perm [2,3,0,1]
+  if (W >= 8) v = dpp_add(v, 0x141);    // row_half_mirror
+  if (W >= 16) v = dpp_add(v, 0x140);   // row_mirror
+  if (W >= 32) v += __shfl_xor(v, 16);
+  return v;
+}
+
 // Force a value to be computed where this statement stands.  The optimiser otherwise sinks arithmetic
 // on loaded registers towards its first use, which can carry it past the issue of the NEXT batch of
 // loads: the in-order vector-memory counter then makes the old value wait for the new loads.

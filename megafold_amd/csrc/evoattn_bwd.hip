@@ -116,8 +116,7 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
         float part = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) part += (float)sdo[i][e] * (float)of[e];
-#pragma unroll
-        for (int m = 1; m < CPR; m <<= 1) part += __shfl_xor(part, m);
+        part = group_sum<CPR>(part);
         sdelta[i] = part;
         sls[i] = __builtin_inff();
         if (dc == 0 && qi < S) {
@@ -446,8 +445,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
 #pragma unroll
         for (int e = 0; e < 8; ++e) part += (float)sa[e] * (float)sb[e];
       }
-#pragma unroll
-      for (int m = 1; m < CPR; m <<= 1) part += __shfl_xor(part, m);
+      part = group_sum<CPR>(part);
       if (sdc == 0) {
         Dpk[buf * 32 + srow] = pack_split<T>(-part);
         if (write_delta && qi < S) p.delta[row_base + qi] = part;

@@ -42,6 +42,10 @@ struct LnParams {
   float* dbeta;        // [K] or null
   float* Gpart;        // [R, K, N] partial x_hat^T dOut
   float* spart;        // [R, N]   partial column sums of dOut
+#ifdef MF_TIMELINE
+  unsigned* tl;        // development aid: cycle stamps of one work-group (see MF_TL in common.h)
+  int tl_block;
+#endif
   int R;               // number of row ranges (partials)
   int64_t rows_per_range;
 };

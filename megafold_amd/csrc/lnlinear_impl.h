@@ -73,6 +73,11 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
   float* rstdL = meanL + 2 * RB;                                   // [2][RB]
   float* csL = rstdL + 2 * RB;                                     // [4 * NTW * 32]
   float* bpL = csL + 4 * NTW * 32;
+  // per-wavefront output tile(s), row-major: results leave the registers with one row per lane and
+  // are stored from here with consecutive lanes on consecutive 16-byte chunks (whole cache lines)
+  constexpr int OSTR = OUTW + 16 / (int)sizeof(T);
+  constexpr int OTILES = (ACT == LN_ACT_SWIGLU_BWD) ? 2 : 1;
+  T* Os = reinterpret_cast<T*>(bpL + 4 * NTW * 32) + (threadIdx.x >> 6) * (OTILES * 32 * OSTR);
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int wn = w % WN, wr = w / WN;
@@ -121,12 +126,14 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
       xr[i] = ld8<T>(X + m * p.K + (8 * dc < p.K ? 8 * dc : 0));
     }
   };
-  auto stash = [&](int64_t rb, int buf) {
+  auto stash = [&](int64_t rb, int buf, bool valid) {
     T* xd = Xs + buf * RB * L::XSTR;
+    float mu_s[PFMAX], rs_s[PFMAX];
 #pragma unroll
     for (int i = 0; i < PFMAX; ++i) {
       const int item = tid + 256 * i;
-      if (item < items) {
+      mu_s[i] = 0.0f; rs_s[i] = 0.0f;
+      if (items % 256 == 0 || item < items) {   // compile-time true for whole multiples: no branch
         const int row = item / CPR, dc = item % CPR;
         const int64_t m = rb * RB + row;
         const bool live = m < p.M && 8 * dc < p.K;
@@ -135,23 +142,73 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
         float s = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) s += to_f(xv[e]);
-#pragma unroll
-        for (int msk = 1; msk < CPR; msk <<= 1) s += __shfl_xor(s, msk);
+        s = group_sum<CPR>(s);
         const float mu = s / (float)p.K;
         float d = 0.0f;
         if (8 * dc < p.K) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) { const float c = to_f(xv[e]) - mu; d += c * c; }
         }
-#pragma unroll
-        for (int msk = 1; msk < CPR; msk <<= 1) d += __shfl_xor(d, msk);
+        d = group_sum<CPR>(d);
         const float rs = __builtin_amdgcn_rsqf(d / (float)p.K + p.eps);
+        mu_s[i] = mu; rs_s[i] = rs;
         if (dc == 0) {
           meanL[buf * RB + row] = mu;
           rstdL[buf * RB + row] = rs;
-          if (ACT != LN_ACT_SWIGLU_BWD && blockIdx.y == 0 && m < p.M) { p.mean[m] = mu; p.rstd[m] = rs; }
         }
       }
+    }
+    // the statistics go to global memory only after every staged register has been consumed: a store
+    // issued between two of them would have to be acknowledged before the second one may be read
+    if (ACT != LN_ACT_SWIGLU_BWD && blockIdx.y == 0 && valid) {
+#pragma unroll
+      for (int i = 0; i < PFMAX; ++i) {
+        const int item = tid + 256 * i;
+        const int64_t m = rb * RB + item / CPR;
+        if (item < items && item % CPR == 0 && m < p.M) { p.mean[m] = mu_s[i]; p.rstd[m] = rs_s[i]; }
+      }
+    }
+  };
+
+  // SwiGLU backward: the incoming gradient of a block is requested one iteration ahead (coalesced:
+  // lane l takes chunk l % DCH of rows l / DCH + j * DRPI) and consumed in that block's epilogue
+  constexpr int DCH = OUTW / 8, DRPI = 64 / DCH, DNL = (ACT == LN_ACT_SWIGLU_BWD) ? 32 / DRPI : 1;
+  frag dpre[DNL];
+  auto fetch_dh = [&](int64_t rbx) {
+    if constexpr (ACT == LN_ACT_SWIGLU_BWD) {
+      const T* dsrc = reinterpret_cast<const T*>(p.dout);
+      const int ch = l % DCH, r0 = l / DCH;
+      const int col = base + 8 * ch < Nhalf ? base + 8 * ch : 0;
+#pragma unroll
+      for (int j = 0; j < DNL; ++j) {
+        int64_t mm = rbx * RB + wr * 32 + r0 + j * DRPI;
+        mm = mm < p.M ? mm : p.M - 1;
+        dpre[j] = ld8<T>(dsrc + mm * Nhalf + col);
+      }
+    }
+  };
+  // flush of one staged output tile: lane l takes chunk l % CH of rows l / CH + j * (64 / CH)
+  auto flush = [&](int64_t rbx, const T* tile, T* gbase, int64_t ld, int col_base, int col_limit) {
+    constexpr int CH = OUTW / 8, RPI = 64 / CH;
+    const int ch = l % CH, r0 = l / CH;
+#pragma unroll 2
+    for (int j = 0; j < 32 / RPI; ++j) {
+      const int row = r0 + j * RPI;
+      const int64_t mm = rbx * RB + wr * 32 + row;
+      const frag v = ld8<T>(tile + row * OSTR + 8 * ch);
+      if (mm < p.M && col_base + 8 * ch < col_limit) st8<T>(gbase + mm * ld + col_base + 8 * ch, v);
+    }
+  };
+  // The results of a block stay in the wavefront's LDS tile and are stored one iteration later,
+  // right after the loads of the block after next have been requested: see the loop.
+  auto flush_block = [&](int64_t rbx) {
+    if constexpr (ACT == LN_ACT_NONE) {
+      flush(rbx, Os, reinterpret_cast<T*>(p.out), p.N, base, p.N);
+    } else if constexpr (ACT == LN_ACT_SWIGLU) {
+      flush(rbx, Os, reinterpret_cast<T*>(p.out), Nhalf, base, Nhalf);
+    } else {
+      flush(rbx, Os, reinterpret_cast<T*>(p.du), p.N, base, Nhalf);
+      flush(rbx, Os + 32 * OSTR, reinterpret_cast<T*>(p.du) + Nhalf, p.N, base, Nhalf);
     }
   };
 
@@ -163,12 +220,18 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
   const int64_t nrb = (p.M + RB - 1) / RB;
   const int64_t G = gridDim.x;
   int64_t rb = blockIdx.x;
-  if (rb < nrb) { fetch(rb); stash(rb, 0); }
+  if (rb < nrb) { fetch(rb); stash(rb, 0, true); }
   if (rb + G < nrb) fetch(rb + G);
+  if (rb < nrb) fetch_dh(rb);
+  // One-time drain: the resident W' registers were loaded above and are first used inside the loop;
+  // without this the compiler guards that use with a wait for ALL vector memory in every iteration.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), other counters untouched
   int it = 0;
   for (; rb < nrb; rb += G, ++it) {
     const int buf = it & 1;
-    __syncthreads();
+    // LDS hand-over only.  __syncthreads() would also wait for the output stores of the previous
+    // iteration to be acknowledged, which nothing here depends on.
+    barrier_keep_vm<63>();
 
     const T* xt = Xs + buf * RB * L::XSTR + (wr * 32 + x) * L::XSTR;
     f32x16 acc[NTW];
@@ -181,29 +244,46 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
       for (int t = 0; t < NTW; ++t) acc[t] = mma(af[t][s], bf, acc[t]);
     }
     const float mu_cur = meanL[buf * RB + wr * 32 + x], rs_cur = rstdL[buf * RB + wr * 32 + x];
-    if (rb + G < nrb) stash(rb + G, buf ^ 1);
+    // unconditional (past the end it moves stale registers into a buffer nobody reads): a branch here
+    // would leave the staged registers "possibly still in flight" for everything that follows
+    stash(rb + G, buf ^ 1, rb + G < nrb);
+    frag dcur[DNL];
+#pragma unroll
+    for (int j = 0; j < DNL; ++j) dcur[j] = dpre[j];
     if (rb + 2 * G < nrb) fetch(rb + 2 * G);
+    if (rb + G < nrb) fetch_dh(rb + G);
+    if (it > 0) flush_block(rb - G);
 
     const int64_t m = rb * RB + wr * 32 + x;
     const float mu = mu_cur, rs = rs_cur;
     const float c0 = -rs * mu;
     const float* csw = csL + (wn * NTW) * 32 + 16 * g;
     const float* bpw = bpL + (wn * NTW) * 32 + 16 * g;
-    if (ACT == LN_ACT_NONE) {
-      T* orow = reinterpret_cast<T*>(p.out) + m * p.N;
+    if constexpr (ACT == LN_ACT_NONE) {
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
         float v[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           v[r] = __builtin_fmaf(acc[t][r], rs, __builtin_fmaf(c0, csw[t * 32 + r], bpw[t * 32 + r]));
-        const int col0 = base + (NTW * 16) * g + 16 * t;
-        if (m < p.M) {
-          if (col0 < p.N) st8<T>(orow + col0, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
-          if (col0 + 8 < p.N) st8<T>(orow + col0 + 8, cvt8<T>(v[8], v[9], v[10], v[11], v[12], v[13], v[14], v[15]));
-        }
+        T* orow = Os + x * OSTR + (NTW * 16) * g + 16 * t;
+        st8<T>(orow, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
+        st8<T>(orow + 8, cvt8<T>(v[8], v[9], v[10], v[11], v[12], v[13], v[14], v[15]));
       }
     } else {
+      frag dh[2 * TH];
+      if constexpr (ACT == LN_ACT_SWIGLU_BWD) {
+        // incoming gradient of h: through the second tile, read back one row per lane
+        const int ch = l % DCH, r0 = l / DCH;
+        T* dtile = Os + 32 * OSTR;
+#pragma unroll
+        for (int j = 0; j < DNL; ++j) st8<T>(dtile + (r0 + j * DRPI) * OSTR + 8 * ch, dcur[j]);
+#pragma unroll
+        for (int th = 0; th < TH; ++th) {
+          dh[2 * th] = ld8<T>(dtile + x * OSTR + (TH * 16) * g + 16 * th);
+          dh[2 * th + 1] = ld8<T>(dtile + x * OSTR + (TH * 16) * g + 16 * th + 8);
+        }
+      }
 #pragma unroll
       for (int th = 0; th < TH; ++th) {
         float a[16], gt[16];
@@ -212,42 +292,35 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
           a[r] = __builtin_fmaf(acc[th][r], rs, __builtin_fmaf(c0, csw[th * 32 + r], bpw[th * 32 + r]));
           gt[r] = __builtin_fmaf(acc[TH + th][r], rs, __builtin_fmaf(c0, csw[(TH + th) * 32 + r], bpw[(TH + th) * 32 + r]));
         }
-        const int col0 = base + (TH * 16) * g + 16 * th;   // column of h (and of dh)
-        if (m < p.M && col0 < Nhalf) {
-          const bool two = col0 + 8 < Nhalf;
-          if (ACT == LN_ACT_SWIGLU) {
-            float h[16];
+        const int lcol = (TH * 16) * g + 16 * th;          // column inside this wavefront's tile
+        if constexpr (ACT == LN_ACT_SWIGLU) {
+          float h[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) h[r] = a[r] * gt[r] * sigmoidf_fast(gt[r]);
-            T* orow = reinterpret_cast<T*>(p.out) + m * Nhalf + col0;
-            st8<T>(orow, cvt8<T>(h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]));
-            if (two) st8<T>(orow + 8, cvt8<T>(h[8], h[9], h[10], h[11], h[12], h[13], h[14], h[15]));
-          } else {
-            // SwiGLU backward on the recomputed pre-activation (fused_transition.py:44-47)
-            const T* drow = reinterpret_cast<const T*>(p.dout) + m * Nhalf + col0;
-            const frag d0 = ld8<T>(drow);
-            const frag d1 = two ? ld8<T>(drow + 8) : frag_zero<T>();
-            float da[16], dg[16];
+          for (int r = 0; r < 16; ++r) h[r] = a[r] * gt[r] * sigmoidf_fast(gt[r]);
+          st8<T>(Os + x * OSTR + lcol, cvt8<T>(h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]));
+          st8<T>(Os + x * OSTR + lcol + 8, cvt8<T>(h[8], h[9], h[10], h[11], h[12], h[13], h[14], h[15]));
+        } else {
+          // SwiGLU backward on the recomputed pre-activation (fused_transition.py:44-47)
+          float da[16], dg[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float dh = to_f(r < 8 ? d0[r & 7] : d1[r & 7]);
-              const float sg = sigmoidf_fast(gt[r]);
-              const float silu = gt[r] * sg;
-              da[r] = dh * silu;
-              dg[r] = dh * a[r] * (sg + silu * (1.0f - sg));
-            }
-            T* urow = reinterpret_cast<T*>(p.du) + m * p.N;
-            st8<T>(urow + col0, cvt8<T>(da[0], da[1], da[2], da[3], da[4], da[5], da[6], da[7]));
-            st8<T>(urow + Nhalf + col0, cvt8<T>(dg[0], dg[1], dg[2], dg[3], dg[4], dg[5], dg[6], dg[7]));
-            if (two) {
-              st8<T>(urow + col0 + 8, cvt8<T>(da[8], da[9], da[10], da[11], da[12], da[13], da[14], da[15]));
-              st8<T>(urow + Nhalf + col0 + 8, cvt8<T>(dg[8], dg[9], dg[10], dg[11], dg[12], dg[13], dg[14], dg[15]));
-            }
+          for (int r = 0; r < 16; ++r) {
+            const float dhv = to_f(r < 8 ? dh[2 * th][r & 7] : dh[2 * th + 1][r & 7]);
+            const float sg = sigmoidf_fast(gt[r]);
+            const float silu = gt[r] * sg;
+            da[r] = dhv * silu;
+            dg[r] = dhv * a[r] * (sg + silu * (1.0f - sg));
           }
+          T* t0 = Os + x * OSTR + lcol;
+          T* t1 = Os + 32 * OSTR + x * OSTR + lcol;
+          st8<T>(t0, cvt8<T>(da[0], da[1], da[2], da[3], da[4], da[5], da[6], da[7]));
+          st8<T>(t0 + 8, cvt8<T>(da[8], da[9], da[10], da[11], da[12], da[13], da[14], da[15]));
+          st8<T>(t1, cvt8<T>(dg[0], dg[1], dg[2], dg[3], dg[4], dg[5], dg[6], dg[7]));
+          st8<T>(t1 + 8, cvt8<T>(dg[8], dg[9], dg[10], dg[11], dg[12], dg[13], dg[14], dg[15]));
         }
       }
     }
   }
+  if (it > 0) flush_block(rb - G);
 }
 
 static int g_num_cu = 0;
@@ -272,9 +345,13 @@ static hipError_t launch_fwd_w(const LnParams& p, hipStream_t stream) {
   const int gy = (NOUT + WN * OUTW - 1) / (WN * OUTW);
   const int64_t nrb = (p.M + RB - 1) / RB;
   int64_t gx = 2LL * num_cu() / gy;
+  if (const char* e = getenv("MF_LN_GXMUL")) gx = (int64_t)atoi(e) * num_cu() / gy;
   if (gx < 1) gx = 1;
   if (gx > nrb) gx = nrb;
-  const size_t smem = (size_t)2 * RB * L::XSTR * sizeof(T) + (size_t)4 * RB * 4 + (size_t)2 * 4 * NTW * 32 * 4;
+  constexpr int OSTR = OUTW + 16 / (int)sizeof(T);
+  constexpr int OTILES = (ACT == LN_ACT_SWIGLU_BWD) ? 2 : 1;
+  const size_t smem = (size_t)2 * RB * L::XSTR * sizeof(T) + (size_t)4 * RB * 4 + (size_t)2 * 4 * NTW * 32 * 4 +
+                      (size_t)4 * OTILES * 32 * OSTR * sizeof(T);
   auto kern = ln_fwd_kernel<T, KP, NTW, ACT, WN>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
