@@ -88,16 +88,51 @@ __global__ void __launch_bounds__(256, 2) ln_fwd_kernel(const LnParams p) {
   const T* X = reinterpret_cast<const T*>(p.x);
 
   // ---- this wavefront's slice of W'^T, resident in registers -----------------------------------
+  // Fetched by the whole work-group with consecutive lanes on consecutive 16-byte chunks of a row
+  // (whole cache lines; a lane-per-row gather of the same bytes takes four times as many L1 requests)
+  // and handed to the owning lanes through LDS, one tile of 32 rows per wavefront at a time.
   frag af[NTW][KS];
   {
-    const int gm = (x >> 2) & 1, rr = 4 * (x >> 3) + (x & 3);
+    T* Wst = reinterpret_cast<T*>(bpL + 4 * NTW * 32);     // [4 * 32][XSTR], aliases the output tiles
+    constexpr int WITEMS = 128 * CPR, WPF = WITEMS / 256;   // 16-byte chunks per staged tile / per thread
+    // all tiles are requested up front where the registers allow it (K <= 128), else tile by tile
+    constexpr bool kBatch = KP <= 128;
+    frag wtmp[kBatch ? NTW : 1][WPF];
+    auto request = [&](int t, frag* dst) {
+#pragma unroll
+      for (int i = 0; i < WPF; ++i) {
+        const int item = tid + 256 * i;
+        const int r = item / CPR, dc = item % CPR;          // staged row: wavefront r / 32, lane row r % 32
+        const int xx = r & 31, wq = r >> 5;
+        const int gm = (xx >> 2) & 1, rr = 4 * (xx >> 3) + (xx & 3);
+        const int b2 = (blockIdx.y * WN + wq % WN) * OUTW;
+        const int col = ln_col<NTW, ACT>(t, gm, rr, b2, Nhalf);
+        const bool ok = ln_col_ok<NTW, ACT>(t, gm, rr, b2, p.N, Nhalf);
+        dst[i] = ld8<T>(Wt + (int64_t)(ok ? col : 0) * KP + 8 * dc);
+      }
+    };
+    if constexpr (kBatch) {
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) request(t, wtmp[t]);
+    }
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      const int col = ln_col<NTW, ACT>(t, gm, rr, base, Nhalf);
-      const bool ok = ln_col_ok<NTW, ACT>(t, gm, rr, base, p.N, Nhalf);
+      if constexpr (!kBatch) request(t, wtmp[0]);
+      const frag* src = wtmp[kBatch ? t : 0];
 #pragma unroll
-      for (int s = 0; s < KS; ++s)
-        af[t][s] = ok ? ld8<T>(Wt + (int64_t)col * KP + (KP / 2) * g + 8 * s) : frag_zero<T>();
+      for (int i = 0; i < WPF; ++i) {
+        const int item = tid + 256 * i;
+        const int r = item / CPR, dc = item % CPR;
+        const int xx = r & 31, wq = r >> 5;
+        const int gm = (xx >> 2) & 1, rr = 4 * (xx >> 3) + (xx & 3);
+        const int b2 = (blockIdx.y * WN + wq % WN) * OUTW;
+        const bool ok = ln_col_ok<NTW, ACT>(t, gm, rr, b2, p.N, Nhalf);
+        st8<T>(Wst + r * L::XSTR + 8 * dc, ok ? src[i] : frag_zero<T>());
+      }
+      __syncthreads();
+#pragma unroll
+      for (int s = 0; s < KS; ++s) af[t][s] = ld8<T>(Wst + (w * 32 + x) * L::XSTR + (KP / 2) * g + 8 * s);
+      __syncthreads();
     }
   }
   // column constants of the work-group's columns: index ((wn * NTW + t) * 2 + g) * 16 + rr
@@ -350,8 +385,11 @@ static hipError_t launch_fwd_w(const LnParams& p, hipStream_t stream) {
   if (gx > nrb) gx = nrb;
   constexpr int OSTR = OUTW + 16 / (int)sizeof(T);
   constexpr int OTILES = (ACT == LN_ACT_SWIGLU_BWD) ? 2 : 1;
+  // the output tiles share their space with the staging area of the resident weights (128 rows)
+  constexpr size_t tail_elems = (size_t)4 * OTILES * 32 * OSTR > (size_t)128 * L::XSTR ? (size_t)4 * OTILES * 32 * OSTR
+                                                                                        : (size_t)128 * L::XSTR;
   const size_t smem = (size_t)2 * RB * L::XSTR * sizeof(T) + (size_t)4 * RB * 4 + (size_t)2 * 4 * NTW * 32 * 4 +
-                      (size_t)4 * OTILES * 32 * OSTR * sizeof(T);
+                      tail_elems * sizeof(T);
   auto kern = ln_fwd_kernel<T, KP, NTW, ACT, WN>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
