@@ -986,7 +986,7 @@ int evo_dbias_chunks(int B, int N, int S, int H, int D, int dtype) {
   const double part_cost = (double)B * H * S * S * 8.0 / 2.0e12 / 1.4e-6;
   int best = 1;
   double best_cost = -1.0;
-  for (int c = 1; c <= 16 && c <= N; ++c) {
+  for (int c = 1; c <= 8 && c <= N; ++c) {     // at most 8 partial buffers: they count as activation memory
     const int rows = (N + c - 1) / c;
     if ((N + rows - 1) / rows != c) continue;
     const long long groups_xcd = ((long long)B * H * c + 7) / 8;

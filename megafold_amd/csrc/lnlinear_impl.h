@@ -444,7 +444,10 @@ template <typename T> hipError_t ln_fwd_dispatch(const LnParams& p, int act, hip
 // =================================================================================================
 // backward: dx
 // =================================================================================================
-template <typename T, int KP>
+// RTW row tiles (of 32 rows) per wavefront share every W' fragment read from LDS, and the work-group
+// streams the whole of W' once per 128 * RTW rows: that stream (from L2, through L1) is as large as
+// dOut itself at RTW = 1, so two tiles per wavefront are used where the registers allow it.
+template <typename T, int KP, int RTW>
 __global__ void __launch_bounds__(256, 2) ln_bwd_dx_kernel(const LnParams p, const T* __restrict__ dY) {
   using frag = frag_t<T>;
   constexpr int KPT = KP < 32 ? 32 : KP;       // rows of the W' operand, padded to whole tiles
@@ -452,7 +455,9 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dx_kernel(const LnParams p, con
   constexpr int NC = 64;                       // columns of N per staged chunk
   constexpr int UNIT = 16 / (int)sizeof(T);
   constexpr int WSTR = ((NC / UNIT) % 2 == 0) ? NC + UNIT : NC;
-  constexpr int PF = (KPT * (NC / 8) + 255) / 256;
+  constexpr int WITEMS = KPT * (NC / 8);
+  constexpr int PF = (WITEMS + 255) / 256;
+  constexpr int RBW = 128 * RTW;               // rows per work-group block
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T* Ws = reinterpret_cast<T*>(smem_raw);      // [2][KPT][WSTR]
@@ -464,123 +469,156 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dx_kernel(const LnParams p, con
   const int N = p.N, K = p.K;
   const int nchunks = (N + NC - 1) / NC;
 
+  // W' chunk staging: loads are only issued here (clamped addresses), padding is applied at the stash
   frag wr_[PF];
   auto fetch_w = [&](int c) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int item = tid + 256 * i;
-      wr_[i] = frag_zero<T>();
-      if (item < KPT * (NC / 8)) {
-        const int k = item / (NC / 8), nc = item % (NC / 8);
-        const int n = c * NC + 8 * nc;
-        if (k < K && n < N) wr_[i] = ld8<T>(Wg + (int64_t)k * N + n);
-      }
+      const int k = (item < WITEMS ? item : 0) / (NC / 8), nc = item % (NC / 8);
+      const int n = c * NC + 8 * nc;
+      wr_[i] = ld8<T>(Wg + (int64_t)(k < K ? k : 0) * N + (n < N ? n : 0));
     }
   };
-  auto stash_w = [&](int buf) {
+  auto stash_w = [&](int c, int buf) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int item = tid + 256 * i;
-      if (item < KPT * (NC / 8)) {
+      if (WITEMS % 256 == 0 || item < WITEMS) {
         const int k = item / (NC / 8), nc = item % (NC / 8);
-        st8<T>(Ws + (buf * KPT + k) * WSTR + 8 * nc, wr_[i]);
+        const bool ok = k < K && c * NC + 8 * nc < N;
+        st8<T>(Ws + (buf * KPT + k) * WSTR + 8 * nc, ok ? wr_[i] : frag_zero<T>());
       }
     }
   };
 
-  const int64_t nrb = (p.M + 127) / 128;
+  const int64_t nrb = (p.M + RBW - 1) / RBW;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-    const int64_t m = rb * 128 + w * 32 + x;
-    const int64_t mc = m < p.M ? m : p.M - 1;
-    const T* dyrow = dY + mc * N;
-    f32x16 acc[KT];
+    int64_t m[RTW], mc[RTW];
+    const T* dyrow[RTW];
+    f32x16 acc[RTW][KT];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) acc[kt] = acc_zero();
+    for (int j = 0; j < RTW; ++j) {
+      m[j] = rb * RBW + (j * 4 + w) * 32 + x;
+      mc[j] = m[j] < p.M ? m[j] : p.M - 1;      // rows past the end work on a copy of the last row, store nothing
+      dyrow[j] = dY + mc[j] * N;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) acc[j][kt] = acc_zero();
+    }
 
-    frag yb[4];
+    frag yb[RTW][4];
     auto fetch_y = [&](int c) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int n = c * NC + 32 * g + 8 * s;
-        yb[s] = (m < p.M && n < N) ? ld8<T>(dyrow + n) : frag_zero<T>();
-      }
+      for (int j = 0; j < RTW; ++j)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const int n = c * NC + 32 * g + 8 * s;
+          yb[j][s] = ld8<T>(dyrow[j] + (n < N ? n : 0));
+        }
     };
     __syncthreads();          // the previous row block is done with both W' buffers
     fetch_w(0);
     fetch_y(0);
-    stash_w(0);
+    stash_w(0, 0);
     __syncthreads();
     for (int c = 0; c < nchunks; ++c) {
       const int buf = c & 1;
-      frag yc[4];
+      frag yc[RTW][4];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) yc[s] = yb[s];
-      const bool more = c + 1 < nchunks;
-      if (more) { fetch_w(c + 1); fetch_y(c + 1); }
+      for (int j = 0; j < RTW; ++j)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const bool ok = c * NC + 32 * g + 8 * s < N;     // only the last chunk of a ragged N
+          yc[j][s] = ok ? yb[j][s] : frag_zero<T>();
+          pin(yc[j][s]);
+        }
+      const int cn = c + 1 < nchunks ? c + 1 : c;          // the last chunk is requested twice: no branch
+      fetch_w(cn);
+      fetch_y(cn);
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const T* wrow = Ws + (buf * KPT + dsel<KPT>(kt, x)) * WSTR + 32 * g;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) acc[kt] = mma(ld8<T>(wrow + 8 * s), yc[s], acc[kt]);
+        for (int s = 0; s < 4; ++s) {
+          const frag wf = ld8<T>(wrow + 8 * s);
+#pragma unroll
+          for (int j = 0; j < RTW; ++j) acc[j][kt] = mma(wf, yc[j][s], acc[j][kt]);
+        }
       }
-      if (more) stash_w(buf ^ 1);
+      stash_w(cn, buf ^ 1);
       __syncthreads();
     }
 
-    // ---- LayerNorm backward on the row this lane owns: register r of tile kt <-> k = (KPT/2) g + 16 kt + r
-    const float mu = p.mean[mc], rs = p.rstd[mc];
-    float xh[KT][16];
-    float s1 = 0.0f, s2 = 0.0f;
+    // ---- LayerNorm backward on the rows this lane owns: register r of tile kt <-> k = (KPT/2) g + 16 kt + r
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int j = 0; j < RTW; ++j) {
+      const float mu = p.mean[mc[j]], rs = p.rstd[mc[j]];
+      float xh[KT][16];
+      float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
-        const frag xv = k0 < K ? ld8<T>(X + mc * K + k0) : frag_zero<T>();
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float v = k0 < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
-          xh[kt][8 * u + e] = v;
-          s1 += v * acc[kt][8 * u + e];
-          s2 += acc[kt][8 * u + e];
-        }
-      }
-    }
-    s1 += __shfl_xor(s1, 32);
-    s2 += __shfl_xor(s2, 32);
-    const float c1 = s1 / (float)K, c2 = s2 / (float)K;
-    if (m < p.M) {
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
+      for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
-          if (k0 < K) {
-            float o[8];
+          const frag xv = k0 < K ? ld8<T>(X + mc[j] * K + k0) : frag_zero<T>();
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (acc[kt][8 * u + e] - (xh[kt][8 * u + e] * c1 + c2)) * rs;
-            st8<T>(dX + m * K + k0, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
+          for (int e = 0; e < 8; ++e) {
+            const float v = k0 < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
+            xh[kt][8 * u + e] = v;
+            s1 += v * acc[j][kt][8 * u + e];
+            s2 += acc[j][kt][8 * u + e];
           }
         }
+      }
+      s1 += __shfl_xor(s1, 32);
+      s2 += __shfl_xor(s2, 32);
+      const float c1 = s1 / (float)K, c2 = s2 / (float)K;
+      if (m[j] < p.M) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
+            if (k0 < K) {
+              float o[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) o[e] = (acc[j][kt][8 * u + e] - (xh[kt][8 * u + e] * c1 + c2)) * rs;
+              st8<T>(dX + m[j] * K + k0, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
+            }
+          }
+      }
     }
   }
 }
 
-template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
+template <typename T, int KP, int RTW>
+static hipError_t launch_dx_r(const LnParams& p, const void* dY, hipStream_t stream) {
   constexpr int KPT = KP < 32 ? 32 : KP;
   constexpr int UNIT = 16 / (int)sizeof(T);
   constexpr int WSTR = ((64 / UNIT) % 2 == 0) ? 64 + UNIT : 64;
   const size_t smem = (size_t)2 * KPT * WSTR * sizeof(T);
-  const int64_t nrb = (p.M + 127) / 128;
+  const int64_t nrb = (p.M + 128 * RTW - 1) / (128 * RTW);
   int64_t gx = 2LL * num_cu();
   if (gx > nrb) gx = nrb;
-  auto kern = ln_bwd_dx_kernel<T, KP>;
+  auto kern = ln_bwd_dx_kernel<T, KP, RTW>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)gx), dim3(256), smem, stream, p, reinterpret_cast<const T*>(dY));
   return hipGetLastError();
+}
+
+// Two row tiles per wavefront halve the W' stream but double the block: the grid runs in whole rounds
+// of 2 * CUs resident work-groups, so the larger block only pays when it does not add a partly
+// filled round (a double block is priced at 1.7 single ones).
+template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2 && KP <= 128) {
+    const int64_t slots = 2LL * num_cu();
+    const int64_t r1 = ((p.M + 127) / 128 + slots - 1) / slots, r2 = ((p.M + 255) / 256 + slots - 1) / slots;
+    if (1.7 * (double)r2 < (double)r1) return launch_dx_r<T, KP, 2>(p, dY, stream);
+  }
+  return launch_dx_r<T, KP, 1>(p, dY, stream);
 }
 
 template <typename T> hipError_t ln_dx_dispatch(const LnParams& p, const void* dY, hipStream_t stream) {
@@ -745,25 +783,32 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
   }
 }
 
-// Sum of the per-range partials in a fixed order.  A work-group owns 64 consecutive float4 groups
-// of the flattened [K, N] matrix; its four 64-thread groups each add a quarter of the ranges and
-// the quarters are combined through LDS.  The result overwrites range 0.  Work-groups past the matrix
-// do the same for the column sums.
+// Sum of the per-range partials in a fixed order.  A work-group owns 16 consecutive float4 groups of
+// the flattened [K, N] matrix; its sixteen 16-thread groups each add every 16th range and the groups
+// are combined through LDS.  The result overwrites range 0.  Work-groups past the matrix do the same
+// for the column sums.
 template <typename T>
 __global__ void __launch_bounds__(256) ln_bwd_reduce_kernel(float* __restrict__ Gpart, float* __restrict__ spart,
                                                             int64_t kn, int N, int R, int g_blocks) {
-  __shared__ f32x4 red[4][64];
-  const int tid = threadIdx.x, c = tid & 63, rg = tid >> 6;
+  // a work-group sums 16 float4 columns; its 16 row groups take every 16th range each, so that all
+  // loads of a thread are independent and in flight together
+  __shared__ f32x4 red[16][16];
+  const int tid = threadIdx.x, c = tid & 15, rg = tid >> 4;
   if ((int)blockIdx.x < g_blocks) {
-    const int64_t e = ((int64_t)blockIdx.x * 64 + c) * 4;
+    const int64_t e = ((int64_t)blockIdx.x * 16 + c) * 4;
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     if (e < kn) {
 #pragma unroll 8
-      for (int r = rg; r < R; r += 4) acc += *reinterpret_cast<const f32x4*>(Gpart + (int64_t)r * kn + e);
+      for (int r = rg; r < R; r += 16) acc += *reinterpret_cast<const f32x4*>(Gpart + (int64_t)r * kn + e);
     }
     red[rg][c] = acc;
     __syncthreads();
-    if (rg == 0 && e < kn) *reinterpret_cast<f32x4*>(Gpart + e) = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+    if (rg == 0 && e < kn) {
+      f32x4 tot = red[0][c];
+#pragma unroll
+      for (int q = 1; q < 16; ++q) tot += red[q][c];    // fixed order
+      *reinterpret_cast<f32x4*>(Gpart + e) = tot;
+    }
   } else {
     const int n = ((int)blockIdx.x - g_blocks) * 256 + tid;
     if (n < N) {
@@ -820,7 +865,7 @@ template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, c
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   const int64_t kn = (int64_t)p.K * p.N;
-  const int g_blocks = (int)((kn / 4 + 63) / 64);
+  const int g_blocks = (int)((kn / 4 + 15) / 16);
   const int s_blocks = (p.N + 255) / 256;
   hipLaunchKernelGGL(ln_bwd_reduce_kernel<T>, dim3((unsigned)(g_blocks + s_blocks)), dim3(256), 0, stream, p.Gpart, p.spart,
                      kn, p.N, p.R, g_blocks);
