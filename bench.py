@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the C3/C4/C5 side measurements")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain device copies of 256 MiB (a reference point for reading "
+                         "FETCH_SIZE / WRITE_SIZE hardware counters of the same run)")
     return ap.parse_args()
 
 
@@ -248,6 +251,13 @@ def main():
         "phase_ms": {n: round(per[n], 5) for n in names},
         "hbm_GBps_at_algorithmic_bytes": round(468.0 / ms_per_step, 1),
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 * 2 ** 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        res["calibration_copy_bytes"] = src.numel()
     if not args.no_extras:
         res.update(side_measurements(torch, max(5, args.steps // 5), 3))
     if not args.no_cpu_baseline:

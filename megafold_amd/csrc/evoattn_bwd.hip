@@ -752,13 +752,21 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   const int G = p.B * p.H * p.n_chunks;
   const int bid = blockIdx.x;
   const int xcd = bid & 7, kq = bid >> 3;
-  const int grp = (kq / R) * 8 + xcd;
+  // Each XCD takes a contiguous run of groups (b, head pair, chunk, head in pair): with H * D 16-bit
+  // values per (row, position) two neighbouring heads share every 128-byte line of Q, K, V and dO, so
+  // they should meet in one L2 (otherwise each XCD fetches the line for half of its bytes).  With an
+  // odd run length some pairs straddle two XCDs; the run length is what balances the device.
+  const int hp = (p.H & 1) ? 1 : 2;
+  const int gpx = (G + 7) / 8;                             // groups per XCD
+  const int grp = xcd * gpx + kq / R;
   if (grp >= G) return;
   const int reg = kq % R;
   const int ib = reg % IB, jb = reg / IB;
-  const int chunk = grp % p.n_chunks;
-  const int bh = grp / p.n_chunks;
-  const int h = bh % p.H, b = bh / p.H;
+  // grp = ((b * (H / hp) + head pair) * n_chunks + chunk) * hp + head inside the pair
+  const int hsub = grp % hp;
+  const int chunk = (grp / hp) % p.n_chunks;
+  const int hb = grp / hp / p.n_chunks;
+  const int h = (hb % (p.H / hp)) * hp + hsub, b = hb / (p.H / hp);
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int S = p.S, D = p.D;
