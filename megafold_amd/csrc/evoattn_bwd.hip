@@ -416,18 +416,32 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
   // fetch_q only ISSUES loads (clamped addresses, no arithmetic on the results): zeroing of padded
   // columns / rows and all conversions happen in stash_q, one step later.
   const int sd0 = 8 * sdc < D ? 8 * sdc : 0;
+  // Per-thread source pointers of the staging loads, set at the start of every key chunk (kept in
+  // vector registers: the scalar file is the scarce one in this kernel).  Group A: Q and LSE.
+  // Group B: dO, and O + nothing in the first chunk (delta = <dO, O> is formed there and stored) or
+  // dO again + the stored delta in later chunks, which saves re-reading O.  Every thread issues the
+  // same three loads, so there is no branch around a load.
+  const T* src_a = nullptr;
+  const T* src_b = nullptr;
+  const float* src_s = nullptr;
+  int64_t str_a = 0, str_b = 0;
+  auto point_q = [&](bool first_chunk) {
+    const bool ga = sgrp != 1;
+    src_a = (ga ? Qg : dOg) + sd0;
+    str_a = ga ? p.q.ss : p.dO.ss;
+    const bool use_o = !ga ? first_chunk : false;
+    src_b = ga ? src_a : (use_o ? Og + sd0 : dOg + sd0);
+    str_b = ga ? str_a : (use_o ? p.o.ss : p.dO.ss);
+    src_s = ((ga || first_chunk) ? p.lse : p.delta) + row_base;
+  };
   auto fetch_q = [&](int it) {
     const int qi = it * 32 + srow;
     const int qc = qi < S ? qi : S - 1;
-    if (sgrp == 0) {
-      sa = ld8<T>(Qg + (int64_t)qc * p.q.ss + sd0);
-      sls = p.lse[row_base + qc];
-    } else if (sgrp == 1) {
-      sa = ld8<T>(dOg + (int64_t)qc * p.dO.ss + sd0);
-      sb = ld8<T>(Og + (int64_t)qc * p.o.ss + sd0);
-    }
+    sa = ld8<T>(src_a + (int64_t)qc * str_a);
+    sb = ld8<T>(src_b + (int64_t)qc * str_b);
+    sls = src_s[qc];
   };
-  auto stash_q = [&](int it, int buf, bool write_delta) {
+  auto stash_q = [&](int it, int buf, bool first_chunk) {
     T* qd = Stage + buf * L::STAGE_ELEMS;
     const int qi = it * 32 + srow;
     const bool dok = 8 * sdc < D;
@@ -446,9 +460,10 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
         for (int e = 0; e < 8; ++e) part += (float)sa[e] * (float)sb[e];
       }
       part = group_sum<CPR>(part);
+      part = first_chunk ? part : sls;
       if (sdc == 0) {
         Dpk[buf * 32 + srow] = pack_split<T>(-part);
-        if (write_delta && qi < S) p.delta[row_base + qi] = part;
+        if (first_chunk && qi < S) p.delta[row_base + qi] = part;
       }
     }
   };
@@ -488,6 +503,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
     };
     load_bias(0);
 
+    point_q(kc == 0);
     fetch_q(0);
     stash_q(0, 0, kc == 0);
     __syncthreads();
