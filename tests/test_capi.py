@@ -107,3 +107,62 @@ def test_python_wrapper_fails_loudly_without_gpu_tensors():
     q = torch.zeros(1, 2, 16, 2, 8)
     with pytest.raises(RuntimeError, match="GPU only"):
         TritonEvoformer(q, q, q, torch.zeros(1, 2, 1, 1, 16), torch.zeros(1, 1, 2, 16, 16))
+
+
+def _ln_args(backward=False):
+    a = _lib.LnLinearArgs()
+    a.M, a.K, a.N = 256, 128, 512
+    a.dtype, a.act, a.eps = _lib.MF_BF16, 0, 1e-5
+    fake = 0x10000  # never dereferenced: every check below fails before a launch
+    for f in ("x", "gamma", "beta", "W", "b", "out", "mean", "rstd"):
+        setattr(a, f, fake)
+    if backward:
+        for f in ("dout", "dx", "dW", "db", "dgamma", "dbeta"):
+            setattr(a, f, fake)
+    return a
+
+
+@pytest.mark.parametrize("mutate, code, text", [
+    (lambda a: setattr(a, "x", None), -1, "x is NULL"),
+    (lambda a: setattr(a, "out", None), -1, "out is NULL"),
+    (lambda a: setattr(a, "M", 0), -2, "positive"),
+    (lambda a: setattr(a, "K", 260), -2, "K=260"),
+    (lambda a: setattr(a, "N", 508), -2, "N=508"),
+    (lambda a: setattr(a, "act", 5), -2, "act 5"),
+    (lambda a: (setattr(a, "act", 1), setattr(a, "N", 520)), -2, "multiple of 16"),
+    (lambda a: setattr(a, "act", 1), -2, "no linear bias"),
+    (lambda a: setattr(a, "dtype", 3), -3, "dtype 3"),
+    (lambda a: setattr(a, "W", 0x10008), -5, "W is not 16-byte aligned"),
+])
+def test_lnlinear_argument_errors(mutate, code, text):
+    lib = _lib.lib()
+    a = _ln_args()
+    mutate(a)
+    assert lib.mf_lnlinear_fwd(C.byref(a)) == code
+    assert text in lib.mf_last_error().decode()
+
+
+def test_lnlinear_workspace_contract():
+    lib = _lib.lib()
+    a = _ln_args()
+    need = lib.mf_lnlinear_fwd_workspace_bytes(C.byref(a))
+    assert need >= 512 * 128 * 2 + 2 * 512 * 4          # transposed scaled weight + two column vectors
+    assert lib.mf_lnlinear_fwd(C.byref(a)) == -6 and "workspace" in lib.mf_last_error().decode()
+    b = _ln_args(backward=True)
+    assert lib.mf_lnlinear_bwd_workspace_bytes(C.byref(b)) >= 128 * 512 * 4
+    assert lib.mf_lnlinear_bwd(C.byref(b)) == -6
+    b.dx = None
+    assert lib.mf_lnlinear_bwd(C.byref(b)) == -1 and "dx is NULL" in lib.mf_last_error().decode()
+    a.K = 260                                            # unsupported shapes report a zero workspace
+    assert lib.mf_lnlinear_fwd_workspace_bytes(C.byref(a)) == 0
+
+
+def test_swiglu_argument_errors():
+    lib = _lib.lib()
+    bf16 = _lib.MF_BF16
+    assert lib.mf_swiglu_fwd(None, 0x10000, 16, 64, bf16, None) == -1
+    assert lib.mf_swiglu_fwd(0x10000, 0x20000, 16, 60, bf16, None) == -2
+    assert lib.mf_swiglu_fwd(0x10000, 0x20000, 16, 64, 9, None) == -3
+    assert lib.mf_swiglu_fwd(0x10004, 0x20000, 16, 64, bf16, None) == -5
+    assert lib.mf_swiglu_bwd(0x10000, 0x20000, None, 16, 64, bf16, None) == -1
+    assert lib.mf_swiglu_bwd(0x10000, 0x20000, 0x30000, 0, 64, bf16, None) == -2
