@@ -591,6 +591,210 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dx_kernel(const LnParams p, con
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// dx for K <= 128 (four k tiles of 32), N <= 16 * NSTEPS * NH <= 1024 and 16-bit element types.  A
+// wavefront owns one k tile and one of NH halves of N and keeps that slice of W' in registers for the
+// whole kernel (A operand), so the only streams are dOut and x in and dx out.  dOut and x rows are
+// fetched coalesced one block ahead, staged in LDS and read by all wavefronts; with NH = 2 the two
+// halves of a k tile are added through LDS; the LayerNorm backward needs row sums over all K, which the
+// k tiles exchange through LDS; dx leaves through an LDS tile so that it is stored in whole lines.
+template <typename T, int NSTEPS, int NH>
+__global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const LnParams p, const T* __restrict__ dY) {
+  using frag = frag_t<T>;
+  static_assert(sizeof(T) == 2, "16-bit element types only");
+  constexpr int NTHR = 256 * NH;
+  constexpr int NP = 16 * NSTEPS * NH;         // padded N
+  constexpr int YSTR = NP + 8, XSTR = 128 + 8;
+  constexpr int YCH = NP / 8;                  // 16-byte chunks per dOut row
+  constexpr int YPF = 32 * YCH / NTHR;         // staged dOut chunks per thread
+  constexpr int XPF = 512 / NTHR;              // staged x chunks per thread
+  static_assert(32 * YCH % NTHR == 0, "whole number of chunks per thread");
+
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T* Ys = reinterpret_cast<T*>(smem_raw);      // [32][YSTR]  dOut block (also used to hand out W')
+  T* Xs = Ys + 32 * YSTR;                      // [32][XSTR]  x block
+  T* Os = Xs + 32 * XSTR;                      // [32][XSTR]  dx block
+  float* part = reinterpret_cast<float*>(Os + 32 * XSTR);   // [4][32][2] per-k-tile row sums
+  float* pair = part + 4 * 32 * 2;                          // [4][16][64] second half's accumulators (NH = 2)
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const int kt = w & 3, nh = w >> 2;
+  const int N = p.N, K = p.K;
+  const T* Wg = reinterpret_cast<const T*>(p.Wg);
+  const T* X = reinterpret_cast<const T*>(p.x);
+  T* dX = reinterpret_cast<T*>(p.dx);
+
+  // ---- resident slice of W' (rows 32 kt .. 32 kt + 31, columns of half nh), handed out through the
+  // dOut staging area one k tile at a time
+  frag af[NSTEPS];
+  for (int ww = 0; ww < 4; ++ww) {
+    frag tmp[YPF];
+#pragma unroll
+    for (int i = 0; i < YPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item / YCH, c = item % YCH;
+      const int k = 32 * ww + r;
+      const bool ok = k < K && 8 * c < N;
+      tmp[i] = ld8<T>(Wg + (int64_t)(ok ? k : 0) * N + (ok ? 8 * c : 0));
+    }
+#pragma unroll
+    for (int i = 0; i < YPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item / YCH, c = item % YCH;
+      const bool ok = 32 * ww + r < K && 8 * c < N;
+      st8<T>(Ys + r * YSTR + 8 * c, ok ? tmp[i] : frag_zero<T>());
+    }
+    __syncthreads();
+    if (kt == ww) {
+      // operand row x holds tile row unperm32(x): accumulator register i of half g <-> k = 32 kt + 16 g + i
+#pragma unroll
+      for (int s = 0; s < NSTEPS; ++s)
+        af[s] = ld8<T>(Ys + unperm32(x) * YSTR + nh * (16 * NSTEPS) + 16 * s + 8 * g);
+    }
+    __syncthreads();
+  }
+
+  // ---- staging registers: dOut and x chunks of the next block, mean / rstd of the lane's row --------
+  frag yr[YPF], xr[XPF];
+  float mu_n = 0.0f, rs_n = 0.0f;
+  auto fetch = [&](int64_t rb) {
+#pragma unroll
+    for (int i = 0; i < YPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item / YCH, c = item % YCH;
+      int64_t m = rb * 32 + r;
+      m = m < p.M ? m : p.M - 1;
+      yr[i] = ld8<T>(dY + m * N + (8 * c < N ? 8 * c : 0));
+    }
+#pragma unroll
+    for (int i = 0; i < XPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item >> 4, c = item & 15;
+      int64_t m = rb * 32 + r;
+      m = m < p.M ? m : p.M - 1;
+      xr[i] = ld8<T>(X + m * K + (8 * c < K ? 8 * c : 0));
+    }
+    int64_t m = rb * 32 + x;
+    m = m < p.M ? m : p.M - 1;
+    mu_n = p.mean[m];
+    rs_n = p.rstd[m];
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < YPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item / YCH, c = item % YCH;
+      st8<T>(Ys + r * YSTR + 8 * c, 8 * c < N ? yr[i] : frag_zero<T>());
+    }
+#pragma unroll
+    for (int i = 0; i < XPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item >> 4, c = item & 15;
+      st8<T>(Xs + r * XSTR + 8 * c, 8 * c < K ? xr[i] : frag_zero<T>());
+    }
+  };
+  // dx block of the previous iteration: consecutive lanes take consecutive 16-byte chunks (whole lines)
+  auto flush = [&](int64_t rb) {
+#pragma unroll
+    for (int i = 0; i < XPF; ++i) {
+      const int item = tid + NTHR * i;
+      const int r = item >> 4, c = item & 15;
+      const int64_t m = rb * 32 + r;
+      const frag v = ld8<T>(Os + r * XSTR + 8 * c);
+      if (m < p.M && 8 * c < K) st8<T>(dX + m * K + 8 * c, v);
+    }
+  };
+
+  const int64_t nrb = (p.M + 31) / 32;
+  const int64_t G = gridDim.x;
+  int64_t rb = blockIdx.x;
+  if (rb < nrb) fetch(rb);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // one-time drain: nothing older than the staged block is in flight
+  int it = 0;
+  for (; rb < nrb; rb += G, ++it) {
+    // (A) everybody is done with the LDS blocks of the previous iteration
+    barrier_keep_vm<63>();
+    stash();
+    const float mu = mu_n, rs = rs_n;
+    fetch(rb + G < nrb ? rb + G : rb);          // the tail repeats the last block rather than branching
+    if (it > 0) flush(rb - G);
+    // (B) this iteration's dOut / x are visible
+    barrier_keep_vm<63>();
+
+    f32x16 acc = acc_zero();
+    const T* yrow = Ys + x * YSTR + nh * (16 * NSTEPS) + 8 * g;
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) acc = mma(af[s], ld8<T>(yrow + 16 * s), acc);
+
+    if constexpr (NH == 2) {
+      // the upper half of N hands its partial products to the lower half's wavefront of the same k tile
+      if (nh == 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) pair[(kt * 16 + i) * 64 + l] = acc[i];
+      }
+      barrier_keep_vm<63>();
+      if (nh == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] += pair[(kt * 16 + i) * 64 + l];
+      }
+    }
+
+    // LayerNorm backward: a lane of half 0 holds w[m][32 kt + 16 g + 0..15]
+    float xh[16];
+    float s1 = 0.0f, s2 = 0.0f;
+    if (nh == 0) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int k0 = 32 * kt + 16 * g + 8 * u;
+        const frag xv = ld8<T>(Xs + x * XSTR + k0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float v = k0 + e < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
+          xh[8 * u + e] = v;
+          s1 += v * acc[8 * u + e];
+          s2 += acc[8 * u + e];
+        }
+      }
+      s1 += __shfl_xor(s1, 32);
+      s2 += __shfl_xor(s2, 32);
+      if (g == 0) { part[(kt * 32 + x) * 2] = s1; part[(kt * 32 + x) * 2 + 1] = s2; }
+    }
+    // (C) row sums of all four k tiles
+    barrier_keep_vm<63>();
+    if (nh == 0) {
+      float t1 = 0.0f, t2 = 0.0f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) { t1 += part[(ww * 32 + x) * 2]; t2 += part[(ww * 32 + x) * 2 + 1]; }
+      const float c1 = t1 / (float)K, c2 = t2 / (float)K;
+      float o[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[i] = (acc[i] - (xh[i] * c1 + c2)) * rs;
+      T* orow = Os + x * XSTR + 32 * kt + 16 * g;
+      st8<T>(orow, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
+      st8<T>(orow + 8, cvt8<T>(o[8], o[9], o[10], o[11], o[12], o[13], o[14], o[15]));
+    }
+  }
+  barrier_keep_vm<63>();
+  if (it > 0) flush(rb - G);
+}
+
+template <typename T, int NSTEPS, int NH>
+static hipError_t launch_dx_res(const LnParams& p, const void* dY, hipStream_t stream) {
+  constexpr int NP = 16 * NSTEPS * NH;
+  const size_t smem = (size_t)(32 * (NP + 8) + 2 * 32 * (128 + 8)) * sizeof(T) + 4 * 32 * 2 * 4 +
+                      (NH == 2 ? (size_t)4 * 16 * 64 * 4 : 0);
+  const int64_t nrb = (p.M + 31) / 32;
+  int64_t gx = (2LL / NH) * num_cu();
+  if (gx > nrb) gx = nrb;
+  auto kern = ln_bwd_dx_res_kernel<T, NSTEPS, NH>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)gx), dim3(256 * NH), smem, stream, p, reinterpret_cast<const T*>(dY));
+  return hipGetLastError();
+}
+
 template <typename T, int KP, int RTW>
 static hipError_t launch_dx_r(const LnParams& p, const void* dY, hipStream_t stream) {
   constexpr int KPT = KP < 32 ? 32 : KP;
@@ -613,6 +817,15 @@ static hipError_t launch_dx_r(const LnParams& p, const void* dY, hipStream_t str
 // of 2 * CUs resident work-groups, so the larger block only pays when it does not add a partly
 // filled round (a double block is priced at 1.7 single ones).
 template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2 && KP == 128) {
+    // register-resident W': K in (64, 128], 64 <= N <= 1024
+    if (p.N >= 64 && !getenv("MF_LN_DX_OLD")) {
+      if (p.N <= 128) return launch_dx_res<T, 8, 1>(p, dY, stream);
+      if (p.N <= 256) return launch_dx_res<T, 16, 1>(p, dY, stream);
+      if (p.N <= 512) return launch_dx_res<T, 32, 1>(p, dY, stream);
+      if (p.N <= 1024) return launch_dx_res<T, 32, 2>(p, dY, stream);   // eight wavefronts, N split in halves
+    }
+  }
   if constexpr (sizeof(T) == 2 && KP <= 128) {
     const int64_t slots = 2LL * num_cu();
     const int64_t r1 = ((p.M + 127) / 128 + slots - 1) / slots, r2 = ((p.M + 255) / 256 + slots - 1) / slots;
