@@ -976,8 +976,13 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
 
 __global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, float* out, int64_t n, int chunks) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    float s = 0.0f;
-    for (int c = 0; c < chunks; ++c) s += part[(int64_t)c * n + i];
+    // chunks <= 8: all loads are issued together, the sum keeps its fixed order
+    float v[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) v[c] = c < chunks ? part[(int64_t)c * n + i] : 0.0f;
+    float s = v[0];
+#pragma unroll
+    for (int c = 1; c < 8; ++c) s += v[c];
     out[i] = s;
   }
 }

@@ -380,7 +380,6 @@ static hipError_t launch_fwd_w(const LnParams& p, hipStream_t stream) {
   const int gy = (NOUT + WN * OUTW - 1) / (WN * OUTW);
   const int64_t nrb = (p.M + RB - 1) / RB;
   int64_t gx = 2LL * num_cu() / gy;
-  if (const char* e = getenv("MF_LN_GXMUL")) gx = (int64_t)atoi(e) * num_cu() / gy;
   if (gx < 1) gx = 1;
   if (gx > nrb) gx = nrb;
   constexpr int OSTR = OUTW + 16 / (int)sizeof(T);
@@ -413,7 +412,7 @@ template <typename T, int KP, int ACT> static hipError_t launch_fwd_k(const LnPa
     if (NOUT <= 64) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
     // the backward form also holds the incoming gradient and two outputs per column: with four tiles
     // per wavefront it would spill registers
-    if (NOUT <= 128 || wide || ACT == LN_ACT_SWIGLU_BWD || getenv("MF_LN_NTW2")) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
+    if (NOUT <= 128 || wide || ACT == LN_ACT_SWIGLU_BWD) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
     return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
   }
 }
@@ -819,7 +818,7 @@ static hipError_t launch_dx_r(const LnParams& p, const void* dY, hipStream_t str
 template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
   if constexpr (sizeof(T) == 2 && KP == 128) {
     // register-resident W': K in (64, 128], 64 <= N <= 1024
-    if (p.N >= 64 && !getenv("MF_LN_DX_OLD")) {
+    if (p.N >= 64) {
       if (p.N <= 128) return launch_dx_res<T, 8, 1>(p, dY, stream);
       if (p.N <= 256) return launch_dx_res<T, 16, 1>(p, dY, stream);
       if (p.N <= 512) return launch_dx_res<T, 32, 1>(p, dY, stream);
@@ -892,51 +891,55 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
 #pragma unroll
   for (int e = 0; e < 8; ++e) colsum[e] = 0.0f;
 
+  // fetch() only issues loads (clamped addresses, nothing touches the results); stash() consumes them
+  // one tile later and applies the padding
   frag xr[PFX], yr[PFY];
   float mur[PFX], rsr[PFX];
   auto fetch = [&](int64_t m0) {
 #pragma unroll
     for (int i = 0; i < PFX; ++i) {
       const int item = tid + 256 * i;
-      xr[i] = frag_zero<T>(); mur[i] = 0.0f; rsr[i] = 0.0f;
-      if (item < XI) {
-        const int row = item / (KPT / 8), dc = item % (KPT / 8);
-        const int64_t m = m0 + row;
-        if (m < m_end && 8 * dc < K) { xr[i] = ld8<T>(X + m * K + 8 * dc); mur[i] = p.mean[m]; rsr[i] = p.rstd[m]; }
-      }
+      const int row = (item < XI ? item : 0) / (KPT / 8), dc = item % (KPT / 8);
+      int64_t m = m0 + row;
+      m = m < m_end ? m : m_end - 1;
+      xr[i] = ld8<T>(X + m * K + (8 * dc < K ? 8 * dc : 0));
+      mur[i] = p.mean[m];
+      rsr[i] = p.rstd[m];
     }
 #pragma unroll
     for (int i = 0; i < PFY; ++i) {
       const int item = tid + 256 * i;
-      yr[i] = frag_zero<T>();
-      if (item < YI) {
-        const int row = item / (CW / 8), cc = item % (CW / 8);
-        const int64_t m = m0 + row;
-        const int n = cb + 8 * cc;
-        if (m < m_end && n < N) yr[i] = ld8<T>(dY + m * N + n);
-      }
+      const int row = (item < YI ? item : 0) / (CW / 8), cc = item % (CW / 8);
+      int64_t m = m0 + row;
+      m = m < m_end ? m : m_end - 1;
+      const int n = cb + 8 * cc;
+      yr[i] = ld8<T>(dY + m * N + (n < N ? n : 0));
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int64_t m0, int buf) {
 #pragma unroll
     for (int i = 0; i < PFX; ++i) {
       const int item = tid + 256 * i;
-      if (item < XI) {
+      if (XI % 256 == 0 || item < XI) {
         const int row = item / (KPT / 8), dc = item % (KPT / 8);
+        const bool live = m0 + row < m_end && 8 * dc < K;
+        const float rs = live ? rsr[i] : 0.0f;            // rows / columns past the end: zero
         float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = (to_f(xr[i][e]) - mur[i]) * rsr[i];   // rows past the end: rs = 0
+        for (int e = 0; e < 8; ++e) v[e] = (to_f(xr[i][e]) - mur[i]) * rs;
         st8<T>(Xs + (buf * RT + row) * XSTR + 8 * dc, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
       }
     }
 #pragma unroll
     for (int i = 0; i < PFY; ++i) {
       const int item = tid + 256 * i;
-      if (item < YI) {
+      if (YI % 256 == 0 || item < YI) {
         const int row = item / (CW / 8), cc = item % (CW / 8);
-        st8<T>(Ys + (buf * RT + row) * YSTR + 8 * cc, yr[i]);
+        const bool live = m0 + row < m_end && cb + 8 * cc < N;
+        const frag yv = live ? yr[i] : frag_zero<T>();
+        st8<T>(Ys + (buf * RT + row) * YSTR + 8 * cc, yv);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) colsum[e] += to_f(yr[i][e]);
+        for (int e = 0; e < 8; ++e) colsum[e] += to_f(yv[e]);
       }
     }
   };
@@ -945,9 +948,10 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
   int it = 0;
   for (int64_t m0 = m_begin; m0 < m_end; m0 += RT, ++it) {
     const int buf = it & 1;
-    stash(buf);
-    __syncthreads();
-    if (m0 + RT < m_end) fetch(m0 + RT);
+    stash(m0, buf);
+    barrier_keep_vm<63>();                              // LDS hand-over only (double-buffered tiles)
+    fetch(m0 + RT < m_end ? m0 + RT : m0);              // the tail repeats the last tile: no branch around loads
+    __builtin_amdgcn_sched_barrier(0);                  // keep the requests here: the scheduler would sink them to their use
     const T* xs = Xs + buf * RT * XSTR;
     const T* ys = Ys + buf * RT * YSTR;
 #pragma unroll
@@ -996,37 +1000,39 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
   }
 }
 
-// Sum of the per-range partials in a fixed order.  A work-group owns 16 consecutive float4 groups of
-// the flattened [K, N] matrix; its sixteen 16-thread groups each add every 16th range and the groups
-// are combined through LDS.  The result overwrites range 0.  Work-groups past the matrix do the same
-// for the column sums.
+// Sum of the per-range partials in a fixed order, first level.  A work-group owns 256 consecutive
+// float4 groups (4 KiB per range: long contiguous reads) of the flattened [K, N] matrix and one of
+// LN_RED_GROUPS interleaved sets of ranges; it adds ranges rq, rq + 8, ... and overwrites range rq.  The
+// finalize kernel adds the remaining (at most 8) ranges.  Work-groups past the matrix sum the column
+// sums completely.
+constexpr int LN_RED_GROUPS = 8;
 template <typename T>
 __global__ void __launch_bounds__(256) ln_bwd_reduce_kernel(float* __restrict__ Gpart, float* __restrict__ spart,
                                                             int64_t kn, int N, int R, int g_blocks) {
-  // a work-group sums 16 float4 columns; its 16 row groups take every 16th range each, so that all
-  // loads of a thread are independent and in flight together
-  __shared__ f32x4 red[16][16];
-  const int tid = threadIdx.x, c = tid & 15, rg = tid >> 4;
-  if ((int)blockIdx.x < g_blocks) {
-    const int64_t e = ((int64_t)blockIdx.x * 16 + c) * 4;
-    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (e < kn) {
+  const int tid = threadIdx.x;
+  if ((int)blockIdx.x < g_blocks * LN_RED_GROUPS) {
+    const int cb = (int)blockIdx.x / LN_RED_GROUPS, rq = (int)blockIdx.x % LN_RED_GROUPS;
+    const int64_t e = ((int64_t)cb * 256 + tid) * 4;
+    if (e < kn && rq < R) {
+      f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll 8
-      for (int r = rg; r < R; r += 16) acc += *reinterpret_cast<const f32x4*>(Gpart + (int64_t)r * kn + e);
-    }
-    red[rg][c] = acc;
-    __syncthreads();
-    if (rg == 0 && e < kn) {
-      f32x4 tot = red[0][c];
-#pragma unroll
-      for (int q = 1; q < 16; ++q) tot += red[q][c];    // fixed order
-      *reinterpret_cast<f32x4*>(Gpart + e) = tot;
+      for (int r = rq; r < R; r += LN_RED_GROUPS) acc += *reinterpret_cast<const f32x4*>(Gpart + (int64_t)r * kn + e);
+      *reinterpret_cast<f32x4*>(Gpart + (int64_t)rq * kn + e) = acc;
     }
   } else {
-    const int n = ((int)blockIdx.x - g_blocks) * 256 + tid;
+    const int n = ((int)blockIdx.x - g_blocks * LN_RED_GROUPS) * 256 + tid;
     if (n < N) {
+      // sixteen independent loads at a time (a one-by-one loop would pay the memory latency R times)
       float sacc = 0.0f;
-      for (int r = 0; r < R; ++r) sacc += spart[(int64_t)r * N + n];
+      int r = 0;
+      for (; r + 16 <= R; r += 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = spart[(int64_t)(r + u) * N + n];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) sacc += v[u];
+      }
+      for (; r < R; ++r) sacc += spart[(int64_t)r * N + n];
       spart[n] = sacc;
     }
   }
@@ -1040,7 +1046,10 @@ __global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) 
   const float bet = p.beta ? to_f(reinterpret_cast<const T*>(p.beta)[k]) : 0.0f;
   float dg = 0.0f, dbt = 0.0f;
   for (int n = tid; n < p.N; n += 256) {
-    const float G = p.Gpart[(int64_t)k * p.N + n];
+    float G = 0.0f;
+    const int64_t kn = (int64_t)p.K * p.N;
+    const int nr = p.R < LN_RED_GROUPS ? p.R : LN_RED_GROUPS;
+    for (int r = 0; r < nr; ++r) G += p.Gpart[(int64_t)r * kn + (int64_t)k * p.N + n];   // fixed order
     const float s = p.spart[n];
     const float wv = to_f(W[(int64_t)k * p.N + n]);
     p.dW[(int64_t)k * p.N + n] = gam * G + bet * s;
@@ -1078,10 +1087,10 @@ template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, c
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   const int64_t kn = (int64_t)p.K * p.N;
-  const int g_blocks = (int)((kn / 4 + 15) / 16);
+  const int g_blocks = (int)((kn / 4 + 255) / 256);
   const int s_blocks = (p.N + 255) / 256;
-  hipLaunchKernelGGL(ln_bwd_reduce_kernel<T>, dim3((unsigned)(g_blocks + s_blocks)), dim3(256), 0, stream, p.Gpart, p.spart,
-                     kn, p.N, p.R, g_blocks);
+  hipLaunchKernelGGL(ln_bwd_reduce_kernel<T>, dim3((unsigned)(g_blocks * LN_RED_GROUPS + s_blocks)), dim3(256), 0, stream,
+                     p.Gpart, p.spart, kn, p.N, p.R, g_blocks);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(ln_bwd_finalize_kernel<T>, dim3((unsigned)p.K), dim3(256), 0, stream, p);
