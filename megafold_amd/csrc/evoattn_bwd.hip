@@ -506,6 +506,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
     point_q(kc == 0);
     fetch_q(0);
     stash_q(0, 0, kc == 0);
+    fetch_q(NT > 1 ? 1 : 0);          // the registers now hold the second query tile
     __syncthreads();
 
     frag kf[KS], kT[2];
@@ -581,8 +582,11 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
       // vector-memory counter retires in order, so a wait for older loads never covers these.  The
       // last step repeats its own loads rather than branching around them.
       __builtin_amdgcn_sched_barrier(0);
+      // staging: the registers hold query tile it + 1, requested a whole step ago; publish it for the
+      // next step and request tile it + 2 into the same registers
+      if (more) stash_q(it + 1, buf ^ 1, kc == 0);
       load_bias(more ? it + 1 : it);
-      fetch_q(more ? it + 1 : it);
+      fetch_q(it + 2 < NT ? it + 2 : NT - 1);
       __builtin_amdgcn_sched_barrier(0);
       if (it > 0) reduce_dq(it - 1);
       fetch_dq_old(it);
@@ -627,7 +631,6 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
         v[0] = dq[4 * c4]; v[1] = dq[4 * c4 + 1]; v[2] = dq[4 * c4 + 2]; v[3] = dq[4 * c4 + 3];
         *reinterpret_cast<f32x4*>(slab + x * L::SSTR + 16 * g + 4 * c4) = v;
       }
-      if (more) stash_q(it + 1, buf ^ 1, kc == 0);
       barrier_keep_vm<63>();   // LDS hand-over only: global loads / stores stay in flight
 
     }
