@@ -977,16 +977,33 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   }
 }
 
-__global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, float* out, int64_t n, int chunks) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    // chunks <= 8: all loads are issued together, the sum keeps its fixed order
-    float v[8];
+// out = sum over chunks of part[c], four elements per thread when `vec` (n a multiple of 4).
+__global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, float* out, int64_t n, int chunks, int vec) {
+  if (vec) {
+    const int64_t n4 = n >> 2;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+      // chunks <= 8: all loads are issued together, the sum keeps its fixed order
+      f32x4 v[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) v[c] = c < chunks ? part[(int64_t)c * n + i] : 0.0f;
-    float s = v[0];
+      for (int c = 0; c < 8; ++c) {
+        const f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+        v[c] = c < chunks ? *reinterpret_cast<const f32x4*>(part + (int64_t)c * n + 4 * i) : z;
+      }
+      f32x4 s = v[0];
 #pragma unroll
-    for (int c = 1; c < 8; ++c) s += v[c];
-    out[i] = s;
+      for (int c = 1; c < 8; ++c) s += v[c];
+      *reinterpret_cast<f32x4*>(out + 4 * i) = s;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+      float v[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) v[c] = c < chunks ? part[(int64_t)c * n + i] : 0.0f;
+      float s = v[0];
+#pragma unroll
+      for (int c = 1; c < 8; ++c) s += v[c];
+      out[i] = s;
+    }
   }
 }
 
@@ -1048,10 +1065,11 @@ template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const Evo
   if (e != hipSuccess) return e;
   if (p.n_chunks > 1) {
     const int64_t n = (int64_t)p.B * p.H * p.S * p.S;
-    int64_t rb = (n + 255) / 256;
+    const int vec = (n & 3) == 0;     // partial buffers and dbias are 16-byte aligned
+    int64_t rb = ((vec ? n >> 2 : n) + 255) / 256;
     if (rb > 2048) rb = 2048;
     hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)rb), dim3(256), 0, stream, p.dbias_part, p.dbias, n,
-                       p.n_chunks);
+                       p.n_chunks, vec);
     e = hipGetLastError();
   }
   return e;

@@ -409,7 +409,13 @@ __global__ void __launch_bounds__(256) bias_prep_kernel(const void* src, int dty
                                                         int64_t sj, float* dst, int H, int S, int nt, float mult,
                                                         int backward_layout, int64_t total4) {
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (int64_t)gridDim.x * 256) {
-    const int l = (int)(idx & 63), c4 = (int)((idx >> 6) & 3);
+    // thread -> float4 of the tile.  Backward layout: in storage order (a lane's four values come from
+    // four rows, consecutive lanes read consecutive keys).  Forward layout: eight consecutive threads
+    // take the 32 consecutive keys of one query row, so that both the reads (128 bytes per row) and the
+    // stores (adjacent chunks for adjacent rows) stay in runs.
+    int l, c4;
+    if (backward_layout) { l = (int)(idx & 63); c4 = (int)((idx >> 6) & 3); }
+    else { const int t = (int)(idx & 255); c4 = t & 3; l = 32 * ((t >> 2) & 1) + (t >> 3); }
     const int64_t tile = idx >> 8;
     const int t1 = (int)(tile % nt);
     const int64_t r1 = tile / nt;
@@ -426,7 +432,7 @@ __global__ void __launch_bounds__(256) bias_prep_kernel(const void* src, int dty
       const int j = backward_layout ? 32 * t0 + x : 32 * t1 + 16 * g + 4 * c4 + e;
       v[e] = (i < S && j < S) ? load_any(src, dtype, b * sb + h * sh + i * si + j * sj) * mult : 0.0f;
     }
-    *reinterpret_cast<f32x4*>(dst + 4 * idx) = v;
+    *reinterpret_cast<f32x4*>(dst + tile * 1024 + 4 * (c4 * 64 + l)) = v;
   }
 }
 
