@@ -48,6 +48,9 @@ SWEEP = [
     ((1000,), 64, 320, torch.bfloat16, False),    # (320, 64)
     ((1200,), 128, 128, torch.bfloat16, False),   # (128, 128)
     ((900,), 128, 8, torch.bfloat16, False),      # (8, 128)
+    ((40000,), 128, 512, torch.bfloat16, True),   # more row blocks than resident work-groups: several iterations each
+    ((33001,), 96, 256, torch.bfloat16, False),   # K padded to 128, ragged last row block, several iterations
+    ((20000,), 128, 1024, torch.float16, False),  # N > 512: eight-wavefront dx kernel
     ((100,), 768, 768, torch.float32, True),      # K beyond the kernels: same eager expression as the reference's fallback
 ]
 
