@@ -350,8 +350,10 @@ __global__ void __launch_bounds__(MAXT) evo_bwd_dqkv_kernel(const EvoParams p) {
 template <typename T> struct RkLayout {
   using L = BwdLayout<T, 32>;
   static constexpr int WAVE_BYTES = L::TR_BYTES + 2 * L::SLAB_BYTES;
-  static size_t smem(int NW) {
-    return (size_t)NW * 32 * L::QSTR * sizeof(T) + (size_t)2 * L::STAGE_ELEMS * sizeof(T) + 128 * 4 +
+  // K chunk, two staged (Q | dO) tiles, the packed -LSE/scale and -delta of every query row, and the
+  // per-wavefront dS tile + dQ slabs
+  static size_t smem(int NW, int NT) {
+    return (size_t)NW * 32 * L::QSTR * sizeof(T) + (size_t)2 * L::STAGE_ELEMS * sizeof(T) + (size_t)NT * 64 * 4 +
            (size_t)NW * WAVE_BYTES;
   }
 };
@@ -369,9 +371,10 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T* Kc = reinterpret_cast<T*>(smem_raw);                                   // [KC][QSTR]
   T* Stage = Kc + KC * L::QSTR;                                             // [2][Q tile | dO tile]
-  unsigned* Lpk = reinterpret_cast<unsigned*>(Stage + 2 * L::STAGE_ELEMS);  // [2][32] packed -LSE/scale
-  unsigned* Dpk = Lpk + 64;                                                 // [2][32] packed -delta
-  unsigned char* Wv = reinterpret_cast<unsigned char*>(Dpk + 64);           // [NW][WAVE_BYTES]
+  const int NT = (p.S + 31) >> 5;
+  unsigned* Lpk = reinterpret_cast<unsigned*>(Stage + 2 * L::STAGE_ELEMS);  // [NT * 32] packed -LSE/scale
+  unsigned* Dpk = Lpk + NT * 32;                                            // [NT * 32] packed -delta
+  unsigned char* Wv = reinterpret_cast<unsigned char*>(Dpk + NT * 32);      // [NW][WAVE_BYTES]
   constexpr int WAVE_BYTES = RkLayout<T>::WAVE_BYTES;
 
   const int bid = blockIdx.x;
@@ -383,7 +386,6 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int S = p.S, D = p.D;
-  const int NT = (S + 31) >> 5;
   const float cexp = p.scale * MF_LOG2E;
   const float inv_scale = 1.0f / p.scale;
 
@@ -405,66 +407,66 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
   const unsigned ones_g = g == 0 ? ones_word<T>() : 0u;
   const frag vaugB = make_aug<T>(ones_g, 0u);
 
-  // Staging of one query tile, split over two groups of 128 threads (one 8-element chunk of one row
-  // each): group A moves Q and -LSE/scale, group B moves dO and forms delta = <dO, O>.  The loads are
-  // issued one step ahead; nothing touches the loaded registers before the stash at the end of the
-  // step, so their latency stays hidden behind the step's matrix products.
-  frag sa, sb;
-  float sls = 0.0f;
-  const int sgrp = tid >> 7;                    // 0: Q, 1: dO / O, >= 2: no staging work
-  const int srow = (tid & 127) / CPR, sdc = tid % CPR;
-  // fetch_q only ISSUES loads (clamped addresses, no arithmetic on the results): zeroing of padded
-  // columns / rows and all conversions happen in stash_q, one step later.
-  const int sd0 = 8 * sdc < D ? 8 * sdc : 0;
-  // Per-thread source pointers of the staging loads, set at the start of every key chunk (kept in
-  // vector registers: the scalar file is the scarce one in this kernel).  Group A: Q and LSE.
-  // Group B: dO, and O + nothing in the first chunk (delta = <dO, O> is formed there and stored) or
-  // dO again + the stored delta in later chunks, which saves re-reading O.  Every thread issues the
-  // same three loads, so there is no branch around a load.
-  const T* src_a = nullptr;
-  const T* src_b = nullptr;
-  const float* src_s = nullptr;
-  int64_t str_a = 0, str_b = 0;
-  auto point_q = [&](bool first_chunk) {
-    const bool ga = sgrp != 1;
-    src_a = (ga ? Qg : dOg) + sd0;
-    str_a = ga ? p.q.ss : p.dO.ss;
-    const bool use_o = !ga ? first_chunk : false;
-    src_b = ga ? src_a : (use_o ? Og + sd0 : dOg + sd0);
-    str_b = ga ? str_a : (use_o ? p.o.ss : p.dO.ss);
-    src_s = ((ga || first_chunk) ? p.lse : p.delta) + row_base;
-  };
-  auto fetch_q = [&](int it) {
-    const int qi = it * 32 + srow;
-    const int qc = qi < S ? qi : S - 1;
-    sa = ld8<T>(src_a + (int64_t)qc * str_a);
-    sb = ld8<T>(src_b + (int64_t)qc * str_b);
-    sls = src_s[qc];
-  };
-  auto stash_q = [&](int it, int buf, bool first_chunk) {
-    T* qd = Stage + buf * L::STAGE_ELEMS;
-    const int qi = it * 32 + srow;
-    const bool dok = 8 * sdc < D;
-    if (sgrp == 0) {
-      st8<T>(qd + srow * L::QSTR + 8 * sdc, dok ? sa : frag_zero<T>());
-      if (sdc == 0) {
-        // rows past S and fully masked rows (LSE = -inf) get +inf: every probability becomes exactly 0
-        const float ls = (qi >= S || sls == -__builtin_inff()) ? __builtin_inff() : sls * inv_scale;
-        Lpk[buf * 32 + srow] = pack_split<T>(-ls);
-      }
-    } else if (sgrp == 1) {
-      st8<T>(qd + 32 * L::QSTR + srow * L::QSTR + 8 * sdc, dok ? sa : frag_zero<T>());
-      float part = 0.0f;
-      if (dok) {
+  // ---- once per work-group: delta = <dO, O> and the packed carrier words of every query row -----
+  // Four threads per row (one 8-element chunk each).  Rows past S and fully masked rows (LSE = -inf)
+  // get LSE = +inf: every probability of such a row becomes exactly 0.
+  {
+    constexpr int PB = 4;                          // rows in flight per thread
+    const int items = NT * 32 * CPR;
+    const int c = tid % CPR;
+    const int cd0 = 8 * c < D ? 8 * c : 0;
+    for (int base = 0; base < items; base += PB * nthr) {
+      frag a[PB], o[PB];
+      float ls[PB];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) part += (float)sa[e] * (float)sb[e];
+      for (int u = 0; u < PB; ++u) {
+        const int row = (base + u * nthr + tid) / CPR;
+        const unsigned rc = (unsigned)(row < S ? row : S - 1);
+        a[u] = ld8<T>(dOg + __umul24(rc, (unsigned)p.dO.ss) + cd0);
+        o[u] = ld8<T>(Og + __umul24(rc, (unsigned)p.o.ss) + cd0);
+        ls[u] = p.lse[row_base + rc];
       }
-      part = group_sum<CPR>(part);
-      part = first_chunk ? part : sls;
-      if (sdc == 0) {
-        Dpk[buf * 32 + srow] = pack_split<T>(-part);
-        if (first_chunk && qi < S) p.delta[row_base + qi] = part;
+#pragma unroll
+      for (int u = 0; u < PB; ++u) {
+        const int row = (base + u * nthr + tid) / CPR;
+        float part = 0.0f;
+        if (8 * c < D) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) part += (float)a[u][e] * (float)o[u][e];
+        }
+        part = group_sum<CPR>(part);
+        if (c == 0 && row < NT * 32) {
+          const float l2 = (row >= S || ls[u] == -__builtin_inff()) ? __builtin_inff() : ls[u] * inv_scale;
+          Lpk[row] = pack_split<T>(-l2);
+          Dpk[row] = pack_split<T>(-part);
+          if (row < S) p.delta[row_base + row] = part;
+        }
       }
+    }
+  }
+
+  // Staging of one query tile: threads 0..127 move Q, threads 128..255 move dO (one 8-element chunk
+  // of one row each).  Loads are issued two steps ahead into two alternating registers (tile t uses
+  // register t & 1) and nothing touches a loaded register before its stash: by then the wait for the
+  // bias tile of the step, which was requested later, has already covered it.
+  frag sa0, sa1;
+  const int sgrp = tid >> 7;                    // 0: Q, 1: dO, >= 2: no staging work
+  const int srow = (tid & 127) / CPR, sdc = tid % CPR;
+  const int sd0 = 8 * sdc < D ? 8 * sdc : 0;
+  // Row strides as 24-bit unsigned values (checked by the launcher): row * stride is then one
+  // full-rate multiply instead of a 64-bit product.
+  const T* const src_a = (sgrp != 1 ? Qg : dOg) + sd0;
+  const unsigned str_a = (unsigned)(sgrp != 1 ? p.q.ss : p.dO.ss);
+  const unsigned dq_ss = (unsigned)p.dq.ss;
+  auto fetch_q = [&](int it, frag& sa) {
+    const int qi = (it < NT ? it : NT - 1) * 32 + srow;
+    const int qc = qi < S ? qi : S - 1;
+    sa = ld8<T>(src_a + __umul24((unsigned)qc, str_a));
+  };
+  auto stash_q = [&](int buf, const frag& sa) {
+    if (sgrp < 2) {
+      T* qd = Stage + buf * L::STAGE_ELEMS + sgrp * 32 * L::QSTR;
+      st8<T>(qd + srow * L::QSTR + 8 * sdc, 8 * sdc < D ? sa : frag_zero<T>());
     }
   };
 
@@ -503,10 +505,10 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
     };
     load_bias(0);
 
-    point_q(kc == 0);
-    fetch_q(0);
-    stash_q(0, 0, kc == 0);
-    fetch_q(NT > 1 ? 1 : 0);          // the registers now hold the second query tile
+    fetch_q(0, sa0);
+    fetch_q(1, sa1);
+    stash_q(0, sa0);
+    fetch_q(2, sa0);
     __syncthreads();
 
     frag kf[KS], kT[2];
@@ -529,15 +531,23 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
     auto fetch_dq_old = [&](int it) {
       if (kc > 0 && reducer) {
         const int qi = it * 32 + rrow;
-        dq_old = *reinterpret_cast<const out4_t*>(dQg + (int64_t)(qi < S ? qi : S - 1) * p.dq.ss + (4 * rc4 < D ? 4 * rc4 : 0));
+        dq_old = *reinterpret_cast<const out4_t*>(dQg + __umul24((unsigned)(qi < S ? qi : S - 1), dq_ss) + (4 * rc4 < D ? 4 * rc4 : 0));
+      }
+    };
+    // reduce_load requests the four first slabs' values of step `it` at the top of the following step,
+    // together with that step's operand reads; reduce_dq finishes the sum after the step's loads
+    // have been issued.
+    f32x4 part[4];
+    auto reduce_load = [&](int it) {
+      if (reducer) {
+        const float* sl0 = reinterpret_cast<const float*>(Wv + L::TR_BYTES) + (it & 1) * (32 * L::SSTR) + rrow * L::SSTR + 4 * rc4;
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) part[ww] = *reinterpret_cast<const f32x4*>(sl0 + ww * (WAVE_BYTES / 4));
       }
     };
     auto reduce_dq = [&](int it) {
       if (reducer) {
         const float* sl0 = reinterpret_cast<const float*>(Wv + L::TR_BYTES) + (it & 1) * (32 * L::SSTR) + rrow * L::SSTR + 4 * rc4;
-        f32x4 part[4];     // NW >= 4: the first four reads are unconditional and issued together
-#pragma unroll
-        for (int ww = 0; ww < 4; ++ww) part[ww] = *reinterpret_cast<const f32x4*>(sl0 + ww * (WAVE_BYTES / 4));
         f32x4 sum = part[0];
 #pragma unroll
         for (int ww = 1; ww < 4; ++ww) sum += part[ww];
@@ -552,14 +562,18 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
             for (int e = 0; e < 4; ++e) o4[e] += (float)dq_old[e];
           }
           out4_t ov = {(T)o4[0], (T)o4[1], (T)o4[2], (T)o4[3]};
-          *reinterpret_cast<out4_t*>(dQg + (int64_t)qi * p.dq.ss + 4 * rc4) = ov;
+          *reinterpret_cast<out4_t*>(dQg + __umul24((unsigned)qi, dq_ss) + 4 * rc4) = ov;
         }
       }
     };
 
-    for (int it = 0; it < NT; ++it) {
+    auto step = [&](const int it, frag& sa) {
       const int buf = it & 1;
       const bool more = it + 1 < NT;
+#ifdef MF_TIMELINE
+      const int tls = ((kc * NW + w) * NT + it) * 8;
+#endif
+      MF_TL(p, tls + 0);
 
       const T* qs = Stage + buf * L::STAGE_ELEMS;
       const T* dos = qs + 32 * L::QSTR;
@@ -570,26 +584,32 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
         qA[s] = ld8<T>(qs + arow * L::QSTR + 16 * g + 8 * s);
         doA[s] = ld8<T>(dos + arow * L::QSTR + 16 * g + 8 * s);
       }
-      const frag qaugA = make_aug<T>(ones_g, g == 0 ? Lpk[buf * 32 + arow] : 0u);
-      const frag doaugA = make_aug<T>(g == 0 ? Dpk[buf * 32 + arow] : 0u, 0u);
+      const frag qaugA = make_aug<T>(ones_g, g == 0 ? Lpk[it * 32 + arow] : 0u);
+      const frag doaugA = make_aug<T>(g == 0 ? Dpk[it * 32 + arow] : 0u, 0u);
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         doT[u] = TrRead<T>::read(dos, L::QSTR, 8 * u + 8 * g, g, l, dsel_chunk<DP>(0, l), dsel<DP>(0, x));
         qT[u] = TrRead<T>::read(qs, L::QSTR, 8 * u + 8 * g, g, l, dsel_chunk<DP>(0, l), dsel<DP>(0, x));
       }
+      if (it > 0) reduce_load(it - 1);
       f32x16 z = mma(qaugA, maugB, bzn);
-      // Everything for the next step is requested here, AFTER the last use of the bias registers: the
-      // vector-memory counter retires in order, so a wait for older loads never covers these.  The
-      // last step repeats its own loads rather than branching around them.
+      MF_TL(p, tls + 1);
+      // Everything for the following steps is requested here, AFTER the last use of the bias registers.
+      // The vector-memory counter retires in order, so the order of issue is chosen such that the
+      // only wait of a step is the one for its bias tile (top of the step): the dQ store of the
+      // previous step first, then the read-back of earlier chunks' dQ (used a step later, after the
+      // next bias wait), the next bias tile, and last the query-tile load that has two steps to land.
       __builtin_amdgcn_sched_barrier(0);
-      // staging: the registers hold query tile it + 1, requested a whole step ago; publish it for the
-      // next step and request tile it + 2 into the same registers
-      if (more) stash_q(it + 1, buf ^ 1, kc == 0);
-      load_bias(more ? it + 1 : it);
-      fetch_q(it + 2 < NT ? it + 2 : NT - 1);
-      __builtin_amdgcn_sched_barrier(0);
+      MF_TL(p, tls + 2);
       if (it > 0) reduce_dq(it - 1);
+      MF_TL(p, tls + 3);
+      // staging: `sa` holds query tile it + 1, requested two steps ago; publish it for the next step
+      // and request tile it + 3 into the same register
+      if (more) stash_q(buf ^ 1, sa);
       fetch_dq_old(it);
+      load_bias(more ? it + 1 : it);
+      fetch_q(it + 3, sa);
+      __builtin_amdgcn_sched_barrier(0);
       f32x16 dp = mma(doaugA, vaugB, acc_zero());
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
@@ -605,6 +625,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
       frag pf[2], dsf[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) { pf[u] = acc_half<T>(z, u); dsf[u] = acc_half<T>(dp, u); }
+      MF_TL(p, tls + 4);
       // dS, rows = keys, through this wavefront's LDS tile and back transposed.  LDS operations of one
       // wavefront execute in program order, which is all the ordering this exchange needs; the dV / dK
       // products run while it is in flight.
@@ -620,6 +641,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
         dk = mma(qT[u], dsf[u], dk);
       }
       __builtin_amdgcn_sched_barrier(0);
+      MF_TL(p, tls + 5);
       f32x16 dq = mma(kT[0], dsT[0], acc_zero());
       dq = mma(kT[1], dsT[1], dq);
 
@@ -631,9 +653,19 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
         v[0] = dq[4 * c4]; v[1] = dq[4 * c4 + 1]; v[2] = dq[4 * c4 + 2]; v[3] = dq[4 * c4 + 3];
         *reinterpret_cast<f32x4*>(slab + x * L::SSTR + 16 * g + 4 * c4) = v;
       }
+      MF_TL(p, tls + 6);
       barrier_keep_vm<63>();   // LDS hand-over only: global loads / stores stay in flight
-
+      MF_TL(p, tls + 7);
+    };
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) once: the loop's own wait counts stay exact
+    // two steps per trip, so that each staging register is named statically; an odd last step runs
+    // after the loop
+    for (int it = 0; it + 1 < NT; it += 2) {
+      step(it, sa1);                       // publishes tile it + 1, requests tile it + 3
+      step(it + 1, sa0);
     }
+    if (NT & 1) step(NT - 1, sa1);
+    reduce_load(NT - 1);
     reduce_dq(NT - 1);
 
     if (j < S) {
@@ -655,7 +687,7 @@ __global__ void __launch_bounds__(MAXT, MINW) evo_bwd_dqkv_rk_kernel(const EvoPa
 
 template <typename T, int MAXT, int MINW>
 static hipError_t launch_dqkv_rk_t(const EvoParams& p, int NW, hipStream_t stream) {
-  const size_t smem = RkLayout<T>::smem(NW);
+  const size_t smem = RkLayout<T>::smem(NW, (p.S + 31) / 32);
   if (smem > 160 * 1024) return hipErrorInvalidValue;
   const long long blocks = (long long)round_up(p.B * p.N, 8) * p.H;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
@@ -733,7 +765,11 @@ template <typename T, int DP> static hipError_t launch_dqkv_d(const EvoParams& p
 
 template <typename T> static hipError_t launch_dqkv_s(const EvoParams& p, hipStream_t stream) {
   if constexpr (sizeof(T) == 2) {
-    if (p.D <= 32) return launch_dqkv_rk<T>(p, stream);
+    // the register-resident variant forms row offsets with 24-bit multiplies
+    auto fits = [&](int64_t ss) { return ss < (1 << 24) && (int64_t)p.S * ss < (1LL << 31); };
+    const bool lds_ok = RkLayout<T>::smem(4, (p.S + 31) / 32) <= 80 * 1024;   // two work-groups per compute unit
+    if (p.D <= 32 && lds_ok && fits(p.q.ss) && fits(p.dO.ss) && fits(p.o.ss) && fits(p.dq.ss))
+      return launch_dqkv_rk<T>(p, stream);
   }
   if (p.D <= 32) return launch_dqkv_d<T, 32>(p, stream);
   if (p.D <= 64) return launch_dqkv_d<T, 64>(p, stream);
