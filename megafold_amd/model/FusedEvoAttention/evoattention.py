@@ -117,8 +117,12 @@ def evoattention_forward(Q, K, V, res_mask, pair_bias):
     return O, lse, (Q, K, V, mask, bias)
 
 
-def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None):
+def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None, out=None):
     """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state.
+
+    ``out = (dQ, dK, dV)``, if given, are the tensors to write (``[B, N, S, H, D]`` in Q's dtype, unit
+    stride on D and 16-byte multiples elsewhere, e.g. column slices of a wider matrix); otherwise
+    contiguous tensors are allocated.
 
     ``phase_hook(name)``, if given, is called before and after each backward phase ("prep", "dqkv",
     "dbias"), which are then enqueued by separate C-ABI calls (used by the benchmark to bracket each
@@ -129,9 +133,15 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phas
     dO = _prep_qkv(dO)
     lib = _lib.lib()
     with torch.cuda.device(Q.device):
-        dQ = torch.empty((B, N, S, H, D), dtype=Q.dtype, device=Q.device)
-        dK = torch.empty_like(dQ)
-        dV = torch.empty_like(dQ)
+        if out is None:
+            dQ = torch.empty((B, N, S, H, D), dtype=Q.dtype, device=Q.device)
+            dK = torch.empty_like(dQ)
+            dV = torch.empty_like(dQ)
+        else:
+            dQ, dK, dV = out
+            for t in out:
+                if tuple(t.shape) != (B, N, S, H, D) or t.dtype != Q.dtype or not _strided_ok(t):
+                    raise ValueError("out tensors must be [B, N, S, H, D] in Q's dtype with kernel-compatible strides")
         dbias = torch.empty((B, 1, H, S, S), dtype=torch.float32, device=Q.device) if need_dbias else None
         a = _lib.EvoAttnArgs()
         _fill_common(a, Q, K, V, mask, bias, O, lse)

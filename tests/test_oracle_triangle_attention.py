@@ -1,0 +1,159 @@
+"""Pins the triangle-attention oracle (CPU) against library routines (nn.LayerNorm, nn.Linear,
+F.scaled_dot_product_attention), explicit per-row loops, identities of the block and finite differences;
+checks the parameter names of the fused module against the reference's state-dict keys."""
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from megafold_amd.model.FusedTriangleAttention import PreLayerNormTriangleAttention
+from oracle import triangle_attention as ota
+
+f64 = torch.float64
+
+# state-dict keys of PreLayerNorm(TriangleAttention(dim, heads, node_type, dim_head=...), dim=dim) in the
+# reference (megafold/model/megafold.py:305-320, 598-615; megafold/model/attention.py:120-158)
+REFERENCE_KEYS = {
+    "norm.weight", "norm.bias", "fn.to_attn_bias.0.weight", "fn.attn.to_q.weight", "fn.attn.to_q.bias",
+    "fn.attn.to_kv.weight", "fn.attn.to_out.weight", "fn.attn.to_gates.weight", "fn.attn.to_gates.bias",
+}
+
+
+def make(b=2, n=7, d=16, heads=2, dh=8, seed=0, masked=2):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=f64)
+    inner = heads * dh
+    params = {
+        "norm.weight": 1 + 0.1 * r(d), "norm.bias": 0.1 * r(d),
+        "fn.to_attn_bias.0.weight": r(heads, d) * d ** -0.5,
+        "fn.attn.to_q.weight": r(inner, d) * d ** -0.5, "fn.attn.to_q.bias": 0.1 * r(inner),
+        "fn.attn.to_kv.weight": r(2 * inner, d) * d ** -0.5,
+        "fn.attn.to_gates.weight": r(inner, d) * d ** -0.5, "fn.attn.to_gates.bias": 0.1 * r(inner) - 1.0,
+        "fn.attn.to_out.weight": r(d, inner) * inner ** -0.5,
+    }
+    x = r(b, n, n, d)
+    mask = torch.ones(b, n, dtype=torch.bool)
+    if masked:
+        mask[:, n - masked:] = False
+        mask[0, 1] = False
+    return x, mask, params
+
+
+def library_composition(x, mask, P, heads, dh, node_type):
+    """The block written with torch.nn modules and the library attention routine, one pair-tensor row at a time."""
+    b, n, _, d = x.shape
+    inner = heads * dh
+    ln = nn.LayerNorm(d).double()
+    to_q, to_kv = nn.Linear(d, inner).double(), nn.Linear(d, 2 * inner, bias=False).double()
+    to_g, to_out, to_b = nn.Linear(d, inner).double(), nn.Linear(inner, d, bias=False).double(), nn.Linear(d, heads, bias=False).double()
+    with torch.no_grad():
+        ln.weight.copy_(P["norm.weight"]); ln.bias.copy_(P["norm.bias"])
+        to_q.weight.copy_(P["fn.attn.to_q.weight"]); to_q.bias.copy_(P["fn.attn.to_q.bias"])
+        to_kv.weight.copy_(P["fn.attn.to_kv.weight"])
+        to_g.weight.copy_(P["fn.attn.to_gates.weight"]); to_g.bias.copy_(P["fn.attn.to_gates.bias"])
+        to_out.weight.copy_(P["fn.attn.to_out.weight"]); to_b.weight.copy_(P["fn.to_attn_bias.0.weight"])
+    xn = ln(x)
+    if node_type == "ending":
+        xn = xn.transpose(1, 2)
+    out = torch.empty(b, n, n, d, dtype=f64)
+    for bi in range(b):
+        bias = to_b(xn[bi]).permute(2, 0, 1)                      # [h, i, j]
+        add = torch.zeros(n, dtype=f64).masked_fill(~mask[bi], float("-inf")) if mask is not None else 0.0
+        for row in range(n):
+            seq = xn[bi, row]                                     # [n, d]
+            q = to_q(seq).view(n, heads, dh).transpose(0, 1)
+            k, v = to_kv(seq).chunk(2, dim=-1)
+            k, v = k.view(n, heads, dh).transpose(0, 1), v.view(n, heads, dh).transpose(0, 1)
+            o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias + add)   # [h, n, dh], scale dh^-0.5
+            o = o.transpose(0, 1).reshape(n, inner)
+            out[bi, row] = to_out(o * torch.sigmoid(to_g(seq)))
+    return out.transpose(1, 2) if node_type == "ending" else out
+
+
+@pytest.mark.parametrize("node_type", ["starting", "ending"])
+@pytest.mark.parametrize("masked", [0, 2])
+def test_forward_matches_library_composition(node_type, masked):
+    x, mask, P = make(masked=masked)
+    got = ota.triangle_attention_forward(x, mask if masked else None, P, 2, 8, node_type)
+    with torch.no_grad():
+        want = library_composition(x, mask if masked else None, P, 2, 8, node_type)
+    torch.testing.assert_close(got, want, rtol=1e-10, atol=1e-12)
+
+
+def test_ending_is_starting_on_the_transposed_pair_tensor():
+    x, mask, P = make(seed=3)
+    end = ota.triangle_attention_forward(x, mask, P, 2, 8, "ending")
+    start_t = ota.triangle_attention_forward(x.transpose(1, 2), mask, P, 2, 8, "starting").transpose(1, 2)
+    torch.testing.assert_close(end, start_t, rtol=1e-12, atol=1e-12)
+
+
+def test_masked_keys_are_inert():
+    x, mask, P = make(seed=4, masked=2)
+    base = ota.triangle_attention_forward(x, mask, P, 2, 8, "starting")
+    x2 = x.clone()
+    jm = x.shape[1] - 1                       # a masked key position in every batch element
+    x2[:, :, jm, :] += torch.linspace(-3, 3, x.shape[-1], dtype=f64)   # keys / values at (row, jm) change, other queries do not
+    pert = ota.triangle_attention_forward(x2, mask, P, 2, 8, "starting")
+    keep = [j for j in range(x.shape[2]) if j != jm]
+    torch.testing.assert_close(pert[:, :, keep], base[:, :, keep], rtol=1e-12, atol=1e-12)
+    assert not torch.allclose(pert[:, :, jm], base[:, :, jm])
+
+
+def test_reference_gate_initialisation_scales_the_output():
+    # to_gates.weight = 0, bias = -2 (attention.py:151-154): every gate equals sigmoid(-2)
+    x, mask, P = make(seed=5)
+    P["fn.attn.to_gates.weight"] = torch.zeros_like(P["fn.attn.to_gates.weight"])
+    P["fn.attn.to_gates.bias"] = torch.full_like(P["fn.attn.to_gates.bias"], -2.0)
+    got = ota.triangle_attention_forward(x, mask, P, 2, 8, "starting")
+    P2 = dict(P)
+    P2["fn.attn.to_gates.bias"] = torch.full_like(P["fn.attn.to_gates.bias"], 40.0)     # gate -> 1
+    ungated = ota.triangle_attention_forward(x, mask, P2, 2, 8, "starting")
+    torch.testing.assert_close(got, ungated * torch.sigmoid(torch.tensor(-2.0, dtype=f64)), rtol=1e-10, atol=1e-12)
+
+
+def test_uniform_attention_when_queries_and_bias_vanish():
+    # q = 0 and bias = 0: every kept key gets the same weight, so the attention output is the mean of the kept values
+    x, mask, P = make(seed=6, masked=2)
+    for k in ("fn.attn.to_q.weight", "fn.attn.to_q.bias", "fn.to_attn_bias.0.weight"):
+        P[k] = torch.zeros_like(P[k])
+    P["fn.attn.to_gates.weight"] = torch.zeros_like(P["fn.attn.to_gates.weight"])
+    P["fn.attn.to_gates.bias"] = torch.full_like(P["fn.attn.to_gates.bias"], 40.0)
+    got = ota.triangle_attention_forward(x, mask, P, 2, 8, "starting")
+    xn = F.layer_norm(x, (16,), P["norm.weight"], P["norm.bias"], 1e-5)
+    v = F.linear(xn, P["fn.attn.to_kv.weight"]).chunk(2, dim=-1)[1]                       # [b, row, j, inner]
+    w = mask.to(f64) / mask.sum(-1, keepdim=True)                                         # [b, j]
+    mean_v = torch.einsum("brjc,bj->brc", v, w)
+    want = F.linear(mean_v, P["fn.attn.to_out.weight"]).unsqueeze(2).expand_as(got)
+    torch.testing.assert_close(got, want, rtol=1e-10, atol=1e-12)
+
+
+def test_gradients_match_finite_differences():
+    x, mask, P = make(b=1, n=4, d=8, heads=2, dh=8, seed=7, masked=1)
+    dout = torch.randn(x.shape, generator=torch.Generator().manual_seed(8), dtype=f64)
+    _, dx, dP = ota.triangle_attention_forward_backward(x, mask, P, dout, 2, 8, "ending")
+    loss = lambda xx, PP: (ota.triangle_attention_forward(xx, mask, PP, 2, 8, "ending") * dout).sum()
+    eps = 1e-6
+    for idx in [(0, 1, 2, 3), (0, 3, 0, 5)]:
+        xp, xm = x.clone(), x.clone()
+        xp[idx] += eps; xm[idx] -= eps
+        assert abs((loss(xp, P) - loss(xm, P)) / (2 * eps) - dx[idx]) < 1e-6
+    for name, idx in [("fn.attn.to_kv.weight", (3, 2)), ("fn.to_attn_bias.0.weight", (1, 4)), ("norm.weight", (5,)),
+                      ("fn.attn.to_gates.bias", (7,)), ("fn.attn.to_out.weight", (2, 9)), ("fn.attn.to_q.bias", (0,))]:
+        Pp, Pm = dict(P), dict(P)
+        Pp[name] = P[name].clone(); Pm[name] = P[name].clone()
+        Pp[name][idx] += eps; Pm[name][idx] -= eps
+        assert abs((loss(x, Pp) - loss(x, Pm)) / (2 * eps) - dP[name][idx]) < 1e-6, name
+
+
+@pytest.mark.parametrize("node_type", ["starting", "ending"])
+def test_fused_module_has_the_reference_parameter_names(node_type):
+    m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type=node_type, dim_head=32, dropout=0.25,
+                                      dropout_type="row" if node_type == "starting" else "col")
+    sd = m.state_dict()
+    assert set(sd.keys()) == REFERENCE_KEYS
+    assert sd["fn.attn.to_kv.weight"].shape == (256, 128) and sd["fn.attn.to_out.weight"].shape == (128, 128)
+    assert sd["fn.to_attn_bias.0.weight"].shape == (4, 128)
+    # reference initialisation of the gate (attention.py:151-154)
+    assert torch.all(sd["fn.attn.to_gates.weight"] == 0) and torch.all(sd["fn.attn.to_gates.bias"] == -2.0)
+    with pytest.raises(RuntimeError):
+        m(torch.zeros(1, 4, 4, 128))          # no CPU path

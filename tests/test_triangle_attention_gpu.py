@@ -1,0 +1,99 @@
+"""GPU parity of the fused pre-LayerNorm triangle-attention block against the CPU oracle: output, input
+gradient and every parameter gradient, both node types, with and without key mask.  bf16 runs are compared
+with the float64 oracle on the same (bf16-rounded) inputs at rtol = atol = 2e-2; fp32 runs at 1e-4 / 1e-5
+relative to the size of each tensor."""
+import pytest
+import torch
+
+from conftest import tol_for
+from megafold_amd.model.FusedTriangleAttention import PreLayerNormTriangleAttention
+from oracle import triangle_attention as ota
+
+pytestmark = pytest.mark.gpu
+
+
+def build(dim, heads, dh, node_type, dtype, seed):
+    torch.manual_seed(seed)
+    m = PreLayerNormTriangleAttention(dim=dim, heads=heads, node_type=node_type, dim_head=dh)
+    g = torch.Generator().manual_seed(seed + 1)
+    with torch.no_grad():
+        for name, p in m.named_parameters():
+            if name == "norm.weight":
+                p.copy_(1 + 0.1 * torch.randn(p.shape, generator=g))
+            elif name.endswith("bias"):
+                p.copy_(0.1 * torch.randn(p.shape, generator=g) - (1.0 if "gates" in name else 0.0))
+            else:
+                p.copy_(torch.randn(p.shape, generator=g) * p.shape[1] ** -0.5)
+    return m.to(dtype)
+
+
+CASES = [
+    # b, n, dim, heads, dh, masked, node_type, dtype
+    (1, 48, 128, 4, 32, 5, "starting", torch.bfloat16),
+    (1, 48, 128, 4, 32, 5, "ending", torch.bfloat16),
+    (2, 37, 128, 4, 32, 0, "starting", torch.bfloat16),      # ragged tiles, no mask, batch of two
+    (1, 77, 64, 2, 16, 9, "ending", torch.float16),
+    (1, 40, 128, 4, 32, 3, "starting", torch.float32),
+    (1, 33, 32, 3, 8, 2, "ending", torch.float32),           # 4*inner + heads = 99 -> padded to 104 columns
+]
+
+
+@pytest.mark.parametrize("b,n,dim,heads,dh,masked,node_type,dtype", CASES)
+def test_block_parity(b, n, dim, heads, dh, masked, node_type, dtype):
+    print("case", b, n, dim, heads, dh, masked, node_type, dtype, flush=True)
+    m = build(dim, heads, dh, node_type, dtype, seed=n)
+    g = torch.Generator().manual_seed(100 + n)
+    x = torch.randn(b, n, n, dim, generator=g).to(dtype)
+    dout = torch.randn(b, n, n, dim, generator=g).to(dtype)
+    mask = None
+    if masked:
+        mask = torch.ones(b, n, dtype=torch.bool)
+        mask[:, n - masked:] = False
+        mask[0, 1] = False
+    params = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    want_out, want_dx, want_dp = ota.triangle_attention_forward_backward(x, mask, params, dout, heads, dh, node_type)
+
+    m = m.cuda()
+    xg = x.cuda().requires_grad_(True)
+    out = m(xg, mask.cuda() if mask is not None else None)
+    out.backward(dout.cuda())
+    tol = tol_for(dtype)
+
+    def close(name, got, want):
+        assert not torch.isnan(got).any(), name
+        got = got.detach().cpu().double()
+        # tolerances are relative to the tensor's scale (gradients of weights sum b*n*n terms)
+        s = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(got / s, want / s, msg=lambda msg: "%s: %s" % (name, msg), **tol)
+
+    close("out", out, want_out)
+    close("dx", xg.grad, want_dx)
+    for name, p in m.named_parameters():
+        close(name, p.grad, want_dp[name])
+
+
+def test_block_loads_a_reference_style_state_dict_and_runs_under_autocast():
+    m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type="starting", dim_head=32).cuda()   # fp32 master weights
+    sd = {k: torch.randn_like(v) * 0.05 for k, v in m.state_dict().items()}
+    m.load_state_dict(sd)
+    x = torch.randn(1, 64, 64, 128, device="cuda", requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = m(x)
+    assert out.dtype == torch.bfloat16 and out.shape == x.shape
+    out.float().square().mean().backward()
+    assert x.grad is not None and x.grad.dtype == torch.float32
+    assert all(p.grad is not None and p.grad.dtype == torch.float32 and torch.isfinite(p.grad).all() for p in m.parameters())
+    want = ota.triangle_attention_forward(x.detach().cpu(), None, {k: v.cpu() for k, v in sd.items()}, 4, 32, "starting")
+    torch.testing.assert_close(out.detach().cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_structured_dropout_shapes():
+    m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type="ending", dim_head=32, dropout=0.5,
+                                      dropout_type="col").cuda().to(torch.bfloat16)
+    x = torch.randn(1, 32, 32, 128, device="cuda", dtype=torch.bfloat16)
+    m.train()
+    y = m(x)
+    dropped = (y == 0).all(dim=2)                # "col" dropout zeroes whole [b, row, :, channel] lines
+    assert dropped.any() and not dropped.all()
+    m.eval()
+    assert not (m(x) == 0).all(dim=2).any()
