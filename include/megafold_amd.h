@@ -14,6 +14,9 @@
  *   mf_lnlinear_fwd       layernorm_linear_forward     megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:351-405
  *   mf_lnlinear_bwd       layernorm_linear_backward    megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:408-474
  *   mf_swiglu_fwd / _bwd  swiglu_forward / _backward   megafold/model/FusedTransition/fused_transition.py:55-93
+ *   mf_sigmoid_gate_fwd / _bwd
+ *                         out * gates.sigmoid() of Attention.forward and its autograd backward
+ *                                                      megafold/model/attention.py:199-203
  *   mf_lnlinear_* with act = MF_ACT_SWIGLU
  *                         LayernormLinear + FusedSwiGLU of FusedTransition.ff[0:2]
  *                                                      megafold/model/FusedTransition/fused_transition.py:128-131
@@ -154,6 +157,31 @@ int mf_lnlinear_bwd(const mf_lnlinear_args* a);
  * ---------------------------------------------------------------------------------------------- */
 int mf_swiglu_fwd(const void* x, void* y, int64_t M, int32_t Dh, int32_t dtype, void* stream);
 int mf_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t M, int32_t Dh, int32_t dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Sigmoid output gate of the attention block (megafold/model/attention.py:199-203):
+ *   forward : a = o * sigmoid(g)
+ *   backward: d_o = da * s,  dg = da * o * s * (1 - s),  a = o * s  (s = sigmoid(g); a may be NULL)
+ * Every operand is a matrix of M rows and C columns (C a multiple of 8) with its own row stride in
+ * elements (>= C, 16-byte multiples), so that g / dg can be column slices of the wider matrix the fused
+ * projections produce.  Outputs must not overlap inputs other than element-for-element.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct {
+  int64_t M;
+  int32_t C;
+  int32_t dtype;
+  const void* o;   int64_t ldo;   /* attention output, heads merged */
+  const void* g;   int64_t ldg;   /* gate pre-activations */
+  void* a;         int64_t lda;   /* o * sigmoid(g): output of forward, optional output of backward */
+  /* backward only */
+  const void* da;  int64_t ldda;  /* gradient of a */
+  void* d_o;       int64_t lddo;  /* gradient of o */
+  void* dg;        int64_t lddg;  /* gradient of g */
+  void* stream;
+} mf_gate_args;
+
+int mf_sigmoid_gate_fwd(const mf_gate_args* a);
+int mf_sigmoid_gate_bwd(const mf_gate_args* a);
 
 #ifdef __cplusplus
 }

@@ -49,6 +49,17 @@ class LnLinearArgs(C.Structure):
     ]
 
 
+class GateArgs(C.Structure):
+    _fields_ = [
+        ("M", C.c_int64), ("C", C.c_int32), ("dtype", C.c_int32),
+        ("o", C.c_void_p), ("ldo", C.c_int64), ("g", C.c_void_p), ("ldg", C.c_int64),
+        ("a", C.c_void_p), ("lda", C.c_int64),
+        ("da", C.c_void_p), ("ldda", C.c_int64), ("d_o", C.c_void_p), ("lddo", C.c_int64),
+        ("dg", C.c_void_p), ("lddg", C.c_int64),
+        ("stream", C.c_void_p),
+    ]
+
+
 # every symbol include/megafold_amd.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "mf_version": (C.c_int, []),
@@ -63,6 +74,8 @@ SYMBOLS = {
     "mf_lnlinear_bwd": (C.c_int, [C.POINTER(LnLinearArgs)]),
     "mf_swiglu_fwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]),
     "mf_swiglu_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]),
+    "mf_sigmoid_gate_fwd": (C.c_int, [C.POINTER(GateArgs)]),
+    "mf_sigmoid_gate_bwd": (C.c_int, [C.POINTER(GateArgs)]),
 }
 
 _lock = threading.Lock()

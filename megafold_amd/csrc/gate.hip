@@ -1,0 +1,147 @@
+// Sigmoid output gate of the attention block, forward and backward, and its C-ABI entry points.
+// Reference statement being replaced: `out = out * gates.sigmoid()` (megafold/model/attention.py:199-203)
+// and what autograd derives from it.  Memory-bound elementwise work: every operand is a matrix of M rows
+// and C columns with its own row stride (so that operands can be column slices of a wider matrix), moved
+// in 8-element chunks (16 bytes for the 16-bit types); consecutive lanes take consecutive chunks of a row.
+#include "../../include/megafold_amd.h"
+#include "capi_common.h"
+#include "common.h"
+
+namespace mf {
+namespace {
+
+__device__ __forceinline__ float gate_sigmoid(float g) {
+  return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-g * MF_LOG2E));
+}
+
+struct GateParams {
+  int64_t M;
+  int C;
+  const void* o; int64_t ldo;
+  const void* g; int64_t ldg;
+  void* a; int64_t lda;
+  const void* da; int64_t ldda;
+  void* d_o; int64_t lddo;
+  void* dg; int64_t lddg;
+};
+
+// a = o * sigmoid(g)
+template <typename T>
+__global__ void __launch_bounds__(256) gate_fwd_kernel(const GateParams p) {
+  const int cpr = p.C / 8;
+  const int64_t total = p.M * cpr;
+  const T* O = reinterpret_cast<const T*>(p.o);
+  const T* G = reinterpret_cast<const T*>(p.g);
+  T* A = reinterpret_cast<T*>(p.a);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    const frag_t<T> ov = ld8<T>(O + m * p.ldo + c);
+    const frag_t<T> gv = ld8<T>(G + m * p.ldg + c);
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (float)ov[e] * gate_sigmoid((float)gv[e]);
+    st8<T>(A + m * p.lda + c, cvt8<T>(r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]));
+  }
+}
+
+// d_o = da * s,  dg = da * o * s * (1 - s),  a = o * s (optional),  s = sigmoid(g)
+template <typename T>
+__global__ void __launch_bounds__(256) gate_bwd_kernel(const GateParams p) {
+  const int cpr = p.C / 8;
+  const int64_t total = p.M * cpr;
+  const T* O = reinterpret_cast<const T*>(p.o);
+  const T* G = reinterpret_cast<const T*>(p.g);
+  const T* DA = reinterpret_cast<const T*>(p.da);
+  T* A = reinterpret_cast<T*>(p.a);
+  T* DO = reinterpret_cast<T*>(p.d_o);
+  T* DG = reinterpret_cast<T*>(p.dg);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    const frag_t<T> ov = ld8<T>(O + m * p.ldo + c);
+    const frag_t<T> gv = ld8<T>(G + m * p.ldg + c);
+    const frag_t<T> dv = ld8<T>(DA + m * p.ldda + c);
+    float ra[8], rd[8], rg[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float s = gate_sigmoid((float)gv[e]);
+      const float ofl = (float)ov[e], dfl = (float)dv[e];
+      ra[e] = ofl * s;
+      rd[e] = dfl * s;
+      rg[e] = dfl * ofl * (s * (1.0f - s));
+    }
+    st8<T>(DO + m * p.lddo + c, cvt8<T>(rd[0], rd[1], rd[2], rd[3], rd[4], rd[5], rd[6], rd[7]));
+    st8<T>(DG + m * p.lddg + c, cvt8<T>(rg[0], rg[1], rg[2], rg[3], rg[4], rg[5], rg[6], rg[7]));
+    if (A) st8<T>(A + m * p.lda + c, cvt8<T>(ra[0], ra[1], ra[2], ra[3], ra[4], ra[5], ra[6], ra[7]));
+  }
+}
+
+unsigned gate_blocks(int64_t total) {
+  int64_t b = (total + 255) / 256;
+  const int64_t cap = 16LL * 256;          // 16 work-groups per compute unit, grid-stride beyond that
+  return (unsigned)(b > cap ? cap : (b < 1 ? 1 : b));
+}
+
+int check_matrix(const char* name, const void* ptr, int64_t ld, int C, int es, bool required) {
+  if (!ptr) return required ? fail(MF_ERR_NULL, "%s is NULL", name) : 0;
+  if (!aligned16(ptr)) return fail(MF_ERR_ALIGN, "%s is not 16-byte aligned", name);
+  const int unit = 16 / es;
+  if (ld < C || ld % unit != 0)
+    return fail(MF_ERR_STRIDE, "%s row stride %lld must be >= C and a multiple of %d elements", name, (long long)ld, unit);
+  return 0;
+}
+
+int check_gate(const mf_gate_args* a, bool backward, GateParams& p) {
+  clear_error();
+  if (!a) return fail(MF_ERR_NULL, "args is NULL");
+  if (a->M <= 0 || a->C <= 0 || a->C % 8 != 0)
+    return fail(MF_ERR_SHAPE, "M and C must be positive and C a multiple of 8 (got %lld, %d)", (long long)a->M, a->C);
+  if (a->dtype != MF_DTYPE_F32 && a->dtype != MF_DTYPE_F16 && a->dtype != MF_DTYPE_BF16)
+    return fail(MF_ERR_DTYPE, "dtype %d unsupported", a->dtype);
+  const int es = dtype_size(a->dtype);
+  int rc;
+  if ((rc = check_matrix("o", a->o, a->ldo, a->C, es, true))) return rc;
+  if ((rc = check_matrix("g", a->g, a->ldg, a->C, es, true))) return rc;
+  if ((rc = check_matrix("a", a->a, a->lda, a->C, es, !backward))) return rc;
+  if (backward) {
+    if ((rc = check_matrix("da", a->da, a->ldda, a->C, es, true))) return rc;
+    if ((rc = check_matrix("d_o", a->d_o, a->lddo, a->C, es, true))) return rc;
+    if ((rc = check_matrix("dg", a->dg, a->lddg, a->C, es, true))) return rc;
+  }
+  p = GateParams{a->M, a->C, a->o, a->ldo, a->g, a->ldg, a->a, a->lda, a->da, a->ldda, a->d_o, a->lddo, a->dg, a->lddg};
+  return 0;
+}
+
+}  // namespace
+}  // namespace mf
+
+using namespace mf;
+
+extern "C" int mf_sigmoid_gate_fwd(const mf_gate_args* a) {
+  GateParams p;
+  int rc = check_gate(a, false, p);
+  if (rc) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const unsigned blocks = gate_blocks(a->M * (a->C / 8));
+  switch (a->dtype) {
+    case MF_DTYPE_BF16: hipLaunchKernelGGL(gate_fwd_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    case MF_DTYPE_F16: hipLaunchKernelGGL(gate_fwd_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL(gate_fwd_kernel<float>, dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int mf_sigmoid_gate_bwd(const mf_gate_args* a) {
+  GateParams p;
+  int rc = check_gate(a, true, p);
+  if (rc) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const unsigned blocks = gate_blocks(a->M * (a->C / 8));
+  switch (a->dtype) {
+    case MF_DTYPE_BF16: hipLaunchKernelGGL(gate_bwd_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    case MF_DTYPE_F16: hipLaunchKernelGGL(gate_bwd_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL(gate_bwd_kernel<float>, dim3(blocks), dim3(256), 0, stream, p); break;
+  }
+  return (int)hipGetLastError();
+}

@@ -1,2 +1,2 @@
 from .triangle_attention import (Attention, Dropout, PreLayerNormTriangleAttention, TriangleAttention,  # noqa: F401
-                                 TriangleAttentionFunction)
+                                 TriangleAttentionFunction, sigmoid_gate_backward, sigmoid_gate_forward)

@@ -22,7 +22,9 @@ What runs, per call:
    copies, no ``repeat`` of the bias over rows (megafold.py:634-640), no transposed copies.
 3. The attention kernels (``mf_evoattn_fwd`` / ``mf_evoattn_bwd``).  Backward writes dQ, dK, dV straight
    into the column slices of dY.
-4. Gate and output projection: ``(O * sigmoid(G)) Wo^T`` with PyTorch's elementwise kernels and GEMM.
+4. The sigmoid gate in one pass each way (``mf_sigmoid_gate_fwd`` / ``mf_sigmoid_gate_bwd``, reading the
+   gate columns of ``Y`` and writing the gate columns of dY in place), the output projection and its two
+   gradients through the BLAS library.
 
 Differences from the reference call path (megafold/model/attention.py:466-492), all on purpose: the key
 mask is a real mask (the reference adds the 0/1 values of ``mask.bfloat16()`` to the logits), and the
@@ -31,18 +33,78 @@ storage to ``[(b n1), h, n2, d]`` without permuting).  Both follow the reference
 """
 from __future__ import annotations
 
+import ctypes as C
 from typing import Optional
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from ... import _lib
 from ..FusedEvoAttention.evoattention import evoattention_backward, evoattention_forward
 from ..FusedLayernormLinear.fused_layernorm_linear import (fused_shape_supported, layernorm_linear_backward,
                                                            layernorm_linear_forward)
 
 __all__ = ["Attention", "Dropout", "PreLayerNormTriangleAttention", "TriangleAttention",
-           "TriangleAttentionFunction"]
+           "TriangleAttentionFunction", "sigmoid_gate_forward", "sigmoid_gate_backward"]
+
+
+def _gate_args(O2d, G):
+    if not (O2d.is_cuda and O2d.dim() == 2 and G.shape == O2d.shape and G.dtype == O2d.dtype):
+        raise ValueError("gate operands must be GPU matrices of one shape and dtype")
+    if O2d.stride(1) != 1 or G.stride(1) != 1:
+        raise ValueError("gate operands need unit stride along the columns")
+    a = _lib.GateArgs()
+    a.M, a.C = O2d.shape
+    a.dtype = _lib.dtype_code(O2d.dtype)
+    a.o, a.ldo = O2d.data_ptr(), O2d.stride(0)
+    a.g, a.ldg = G.data_ptr(), G.stride(0)
+    a.stream = torch.cuda.current_stream(O2d.device).cuda_stream
+    return a
+
+
+def sigmoid_gate_forward(O2d: torch.Tensor, G: torch.Tensor) -> torch.Tensor:
+    """``O2d * sigmoid(G)`` (megafold/model/attention.py:199-203) in one pass; ``G`` may be a column slice."""
+    a = _gate_args(O2d, G)
+    with torch.cuda.device(O2d.device):
+        A = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device)
+        a.a, a.lda = A.data_ptr(), A.stride(0)
+        _lib.check(_lib.lib().mf_sigmoid_gate_fwd(C.byref(a)), "mf_sigmoid_gate_fwd")
+    return A
+
+
+def sigmoid_gate_backward(dA: torch.Tensor, O2d: torch.Tensor, G: torch.Tensor, dG_out: torch.Tensor):
+    """Returns ``(dO, A)`` and writes the gate gradient into ``dG_out`` (may be a column slice):
+    ``dO = dA * s``, ``dG = dA * O * s * (1 - s)``, ``A = O * s`` with ``s = sigmoid(G)``."""
+    a = _gate_args(O2d, G)
+    if dA.shape != O2d.shape or dA.dtype != O2d.dtype or dG_out.shape != O2d.shape or dG_out.dtype != O2d.dtype:
+        raise ValueError("gate gradients must match the operands' shape and dtype")
+    dA = dA if dA.stride(1) == 1 else dA.contiguous()
+    with torch.cuda.device(O2d.device):
+        dO = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device)
+        A = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device)
+        a.a, a.lda = A.data_ptr(), A.stride(0)
+        a.da, a.ldda = dA.data_ptr(), dA.stride(0)
+        a.d_o, a.lddo = dO.data_ptr(), dO.stride(0)
+        a.dg, a.lddg = dG_out.data_ptr(), dG_out.stride(0)
+        _lib.check(_lib.lib().mf_sigmoid_gate_bwd(C.byref(a)), "mf_sigmoid_gate_bwd")
+    return dO, A
+
+
+def _tall_skinny_tn(X: torch.Tensor, Y: torch.Tensor) -> torch.Tensor:
+    """``X^T Y`` for X ``[M, p]``, Y ``[M, q]`` with M much larger than p, q (a weight gradient): the long
+    axis is split into slices that run as one batched GEMM and are then summed in fp32, which fills the
+    device where a single [p, M] x [M, q] product would run on a handful of work-groups."""
+    M = X.shape[0]
+    split = 1
+    for cand in (256, 128, 64, 32, 16, 8, 4, 2):
+        if M % cand == 0 and M // cand >= 256:
+            split = cand
+            break
+    if split == 1:
+        return X.t() @ Y
+    part = torch.bmm(X.view(split, M // split, X.shape[1]).transpose(1, 2), Y.view(split, M // split, Y.shape[1]))
+    return part.sum(0, dtype=torch.float32).to(X.dtype)
 
 
 def _views(Y: torch.Tensor, b: int, n: int, heads: int, dh: int):
@@ -85,7 +147,7 @@ class TriangleAttentionFunction(torch.autograd.Function):
             mask5 = mask.to(torch.bool).view(b, 1, 1, 1, n)
         O, lse, (Qs, Ks, Vs, masks, biass) = evoattention_forward(Q, K, V, mask5, Bv)
         O2d = O.view(b * n * n, inner)
-        A = O2d * torch.sigmoid(G)
+        A = sigmoid_gate_forward(O2d, G)
         out = F.linear(A, Wo.to(dt))
         ctx.save_for_backward(x2d, Y, O, lse, Mean, RSTD, masks, Wc, ln_w, ln_b, Wo)
         ctx.dims = (b, n, d, heads, dim_head, pad)
@@ -103,13 +165,12 @@ class TriangleAttentionFunction(torch.autograd.Function):
         dout2d = dout.to(dt).reshape(M, d)
         Q, K, V, G, Bv = _views(Y, b, n, heads, dh)
         O2d = O.view(M, inner)
-        sg = torch.sigmoid(G)
-        dWo = dout2d.t() @ (O2d * sg)                     # [d, inner]
         dA = dout2d @ Wo.to(dt)                           # [M, inner]
         dY = torch.empty_like(Y)
         dQ, dK, dV, dG, dBv = _views(dY, b, n, heads, dh)
-        dO = (dA * sg).view(b, n, n, heads, dh)
-        dG.copy_(dA * O2d * (sg * (1.0 - sg)))
+        dO, A = sigmoid_gate_backward(dA, O2d, G, dG)
+        dWo = _tall_skinny_tn(dout2d, A)                  # [d, inner]
+        dO = dO.view(b, n, n, heads, dh)
         _, _, _, dbias = evoattention_backward(dO, Q, K, V, mask5, Bv, O, lse, True, out=(dQ, dK, dV))
         dY.as_strided((b, heads, n, n), (n * n * Nt, 1, n * Nt, Nt), dY.storage_offset() + 4 * inner).copy_(dbias[:, 0])
         if pad:

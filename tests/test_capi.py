@@ -166,3 +166,52 @@ def test_swiglu_argument_errors():
     assert lib.mf_swiglu_fwd(0x10004, 0x20000, 16, 64, bf16, None) == -5
     assert lib.mf_swiglu_bwd(0x10000, 0x20000, None, 16, 64, bf16, None) == -1
     assert lib.mf_swiglu_bwd(0x10000, 0x20000, 0x30000, 0, 64, bf16, None) == -2
+
+
+def _gate_args():
+    a = _lib.GateArgs()
+    a.M, a.C, a.dtype = 64, 128, _lib.MF_BF16
+    a.o, a.g, a.a = 0x10000, 0x20000, 0x30000          # never dereferenced: every check fails before a launch
+    a.da, a.d_o, a.dg = 0x40000, 0x50000, 0x60000
+    a.ldo = a.lda = a.ldda = a.lddo = 128
+    a.ldg = a.lddg = 520
+    return a
+
+
+@pytest.mark.parametrize("mutate,code,text", [
+    (lambda a: setattr(a, "C", 100), -2, "multiple of 8"),
+    (lambda a: setattr(a, "M", 0), -2, "positive"),
+    (lambda a: setattr(a, "dtype", 3), -3, "dtype"),
+    (lambda a: setattr(a, "g", None), -1, "g is NULL"),
+    (lambda a: setattr(a, "o", 0x10008), -5, "o is not 16-byte aligned"),
+    (lambda a: setattr(a, "ldg", 516), -4, "g row stride"),
+    (lambda a: setattr(a, "ldo", 64), -4, "o row stride"),
+])
+def test_gate_argument_errors(mutate, code, text):
+    lib = _lib.lib()
+    a = _gate_args()
+    mutate(a)
+    assert lib.mf_sigmoid_gate_fwd(C.byref(a)) == code
+    assert text in lib.mf_last_error().decode()
+    assert lib.mf_sigmoid_gate_bwd(C.byref(a)) == code
+
+
+def test_gate_backward_needs_its_gradient_operands():
+    lib = _lib.lib()
+    a = _gate_args()
+    a.dg = None
+    assert lib.mf_sigmoid_gate_bwd(C.byref(a)) == -1 and "dg is NULL" in lib.mf_last_error().decode()
+    a = _gate_args()
+    a.a = None                                           # optional in backward, required in forward
+    assert lib.mf_sigmoid_gate_fwd(C.byref(a)) == -1 and "a is NULL" in lib.mf_last_error().decode()
+    assert lib.mf_sigmoid_gate_fwd(None) == -1
+
+
+def test_gate_struct_layout_matches_header(tmp_path):
+    src = tmp_path / "g.c"
+    src.write_text('#include <stdio.h>\n#include "megafold_amd.h"\nint main(void){printf("%zu %zu %zu\\n", '
+                   'sizeof(mf_gate_args), offsetof(mf_gate_args, da), offsetof(mf_gate_args, stream)); return 0;}\n')
+    exe = tmp_path / "g"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    a, b, c = map(int, subprocess.run([str(exe)], capture_output=True, text=True).stdout.split())
+    assert (a, b, c) == (C.sizeof(_lib.GateArgs), _lib.GateArgs.da.offset, _lib.GateArgs.stream.offset)

@@ -97,3 +97,29 @@ def test_structured_dropout_shapes():
     assert dropped.any() and not dropped.all()
     m.eval()
     assert not (m(x) == 0).all(dim=2).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,C,ld", [(1000, 128, 520), (37, 24, 104), (4096, 64, 64)])
+def test_sigmoid_gate_kernels(dtype, M, C, ld):
+    """mf_sigmoid_gate_fwd / _bwd against torch.sigmoid and autograd in float64; the gate operands are
+    column slices of a wider matrix, as in the fused block."""
+    from megafold_amd.model.FusedTriangleAttention import sigmoid_gate_backward, sigmoid_gate_forward
+    g = torch.Generator().manual_seed(M + C)
+    O = torch.randn(M, C, generator=g).to(dtype)
+    Y = (2 * torch.randn(M, ld, generator=g)).to(dtype)
+    dA = torch.randn(M, C, generator=g).to(dtype)
+    off = ld - C
+    o64, g64 = O.double().requires_grad_(True), Y[:, off:].double().requires_grad_(True)
+    a64 = o64 * torch.sigmoid(g64)
+    do64, dg64 = torch.autograd.grad(a64, [o64, g64], dA.double())
+    Og, Yg = O.cuda(), Y.cuda()
+    tol = tol_for(dtype)
+    A = sigmoid_gate_forward(Og, Yg[:, off:])
+    torch.testing.assert_close(A.cpu().double(), a64.detach(), **tol)
+    dY = torch.full_like(Yg, 7.0)
+    dO, A2 = sigmoid_gate_backward(dA.cuda(), Og, Yg[:, off:], dY[:, off:])
+    torch.testing.assert_close(A2, A, rtol=0, atol=0)
+    torch.testing.assert_close(dO.cpu().double(), do64, **tol)
+    torch.testing.assert_close(dY[:, off:].cpu().double(), dg64, **tol)
+    assert torch.all(dY[:, :off] == 7.0)        # columns outside the slice are untouched
