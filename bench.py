@@ -33,8 +33,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # the device needs some tens of milliseconds of load before its clocks settle: 100 warm-up steps
+    # (about 40 ms) keep the timed region in the steady state
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the C3/C4/C5 side measurements")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -152,7 +154,45 @@ def side_measurements(torch, steps, warmup):
     torch.cuda.synchronize()
     out["c5_peak_act_mib"] = round((torch.cuda.max_memory_allocated() - base) / 2 ** 20, 1)
     out["c5_bound_mib"] = 4 * 144 + 3 * 9
+    del c5, q, k, v, bias, o
+    torch.cuda.empty_cache()
+    out["triangle_attention_block"] = triangle_block(torch, steps, warmup)
     return out
+
+
+def triangle_block(torch, steps, warmup):
+    """fwd / bwd ms of the fused pre-LayerNorm triangle-attention block on a [1, 384, 384, 128] bf16 pair
+    tensor (heads 4 x 32, last 38 keys masked), both node types; autograd end to end, parameters in bf16."""
+    from megafold_amd.model.FusedTriangleAttention import PreLayerNormTriangleAttention
+    n, res = 384, {}
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda().requires_grad_()
+    dout = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda()
+    mask = torch.ones(1, n, dtype=torch.bool, device="cuda")
+    mask[:, n - 38:] = False
+    for node_type in ("starting", "ending"):
+        m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type=node_type, dim_head=32).cuda().to(torch.bfloat16)
+        with torch.no_grad():
+            for p in m.parameters():
+                p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(p.dtype))
+        evs = []
+        for i in range(warmup + steps):       # no host synchronisation inside: launches stay ahead of the GPU
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+            e[0].record()
+            out = m(x, mask)
+            e[1].record()
+            out.backward(dout)
+            e[2].record()
+            x.grad = None
+            for p in m.parameters():
+                p.grad = None
+            if i >= warmup:
+                evs.append(e)
+        torch.cuda.synchronize()
+        tf = [e[0].elapsed_time(e[1]) for e in evs]
+        tb = [e[1].elapsed_time(e[2]) for e in evs]
+        res[node_type] = {"fwd_ms": round(median(tf), 4), "bwd_ms": round(median(tb), 4)}
+    return res
 
 
 def main():
@@ -259,7 +299,7 @@ def main():
         torch.cuda.synchronize()
         res["calibration_copy_bytes"] = src.numel()
     if not args.no_extras:
-        res.update(side_measurements(torch, max(5, args.steps // 5), 3))
+        res.update(side_measurements(torch, max(5, min(40, args.steps // 5)), 5))
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(inp, fl["total"])
     else:
