@@ -407,6 +407,10 @@ template <typename T, int KP, int ACT> static hipError_t launch_fwd_k(const LnPa
     if (NOUT <= 32) return launch_fwd_w<T, KP, 1, ACT, 1>(p, stream);
     if (NOUT <= 128) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
     if (NOUT <= 256 || wide) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
+    // 512-column slabs, unless 256-column slabs pad N up by less and their last slab is at least a quarter
+    // full (measured at M = 147456, K = 128: N = 640 70 against 78 us; N = 520 is better off with 512)
+    const int pad512 = (NOUT + 511) / 512 * 512, pad256 = (NOUT + 255) / 256 * 256;
+    if (pad256 < pad512 && NOUT - (pad256 - 256) >= 64) return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
     return launch_fwd_w<T, KP, 4, ACT, 4>(p, stream);
   } else {
     if (NOUT <= 64) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
