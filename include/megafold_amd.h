@@ -17,6 +17,9 @@
  *   mf_sigmoid_gate_fwd / _bwd
  *                         out * gates.sigmoid() of Attention.forward and its autograd backward
  *                                                      megafold/model/attention.py:199-203
+ *   mf_trimul_pack_fwd / _bwd, mf_channels_last_to_first / _first_to_last
+ *                         glu, chunk, mask and the operand layouts of the einsum in TriangleMultiplication.forward
+ *                                                      megafold/model/megafold.py:474-483
  *   mf_lnlinear_* with act = MF_ACT_SWIGLU
  *                         LayernormLinear + FusedSwiGLU of FusedTransition.ff[0:2]
  *                                                      megafold/model/FusedTransition/fused_transition.py:128-131
@@ -182,6 +185,45 @@ typedef struct {
 
 int mf_sigmoid_gate_fwd(const mf_gate_args* a);
 int mf_sigmoid_gate_bwd(const mf_gate_args* a);
+
+/* ------------------------------------------------------------------------------------------------
+ * Layout moves of the triangle-multiplication block (megafold/model/megafold.py:474-483).  The
+ * contraction  out[i,j,c] = sum_k left[i,k,c] * right[j,k,c]  ("outgoing";  "incoming" is
+ * sum_k left[k,j,c] * right[k,i,c])  is a batch of dh independent n x n x n products, so its operands are
+ * moved from channel-last rows to channel-first matrices  p[which][b][c][o][q]  with row stride and row
+ * count np (a multiple of 8, >= n; positions q >= n of written rows are zero, rows o >= n are not
+ * touched).  With  out_c = p[0][b][c] * p[1][b][c]^T  as the batched product:
+ *   outgoing: transposed = 0, swap = 0   p[0][c][i][k] = left[i,k,c],  p[1][c][j][k] = right[j,k,c]
+ *   incoming: transposed = 1, swap = 1   p[0][c][i][k] = right[k,i,c], p[1][c][j][k] = left[k,j,c]
+ * i.e. the channel-last row of position (o, q) is row o*n + q (transposed = 0) or q*n + o (transposed = 1),
+ * and swap exchanges which of the two channel halves lands in p[0].
+ *
+ *   mf_trimul_pack_fwd        y [B*n*n, ldy >= 4*dh]: columns [0,2dh) values, [2dh,4dh) gates;
+ *                             (left | right) = y[:, :2dh] * sigmoid(y[:, 2dh:4dh]) * mask[b,o] * mask[b,q] -> p
+ *   mf_trimul_pack_bwd        p holds the gradients of the two matrices; writes the gradients of the value
+ *                             and gate columns into dy [B*n*n, lddy >= 4*dh] (y as in forward)
+ *   mf_channels_last_to_first y [B*n*n, ldy >= dh] -> p[0] (one matrix set; mask, if given, is applied)
+ *   mf_channels_first_to_last p[0] -> dy [B*n*n, lddy >= dh]
+ * dh must make the moved row 64, 128 or 256 channels wide (2*dh for the pack forms, dh for the plain ones).
+ * mask: [B, n] bytes (non-zero = keep) or NULL.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct {
+  int32_t B, n, np, dh;
+  int32_t dtype;
+  int32_t transposed;
+  int32_t swap;
+  int32_t reserved0;
+  const void* y;  int64_t ldy;
+  void* dy;       int64_t lddy;
+  const void* mask;
+  void* p;
+  void* stream;
+} mf_trimul_args;
+
+int mf_trimul_pack_fwd(const mf_trimul_args* a);
+int mf_trimul_pack_bwd(const mf_trimul_args* a);
+int mf_channels_last_to_first(const mf_trimul_args* a);
+int mf_channels_first_to_last(const mf_trimul_args* a);
 
 #ifdef __cplusplus
 }

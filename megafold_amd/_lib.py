@@ -60,6 +60,15 @@ class GateArgs(C.Structure):
     ]
 
 
+class TriMulArgs(C.Structure):
+    _fields_ = [
+        ("B", C.c_int32), ("n", C.c_int32), ("np", C.c_int32), ("dh", C.c_int32),
+        ("dtype", C.c_int32), ("transposed", C.c_int32), ("swap", C.c_int32), ("reserved0", C.c_int32),
+        ("y", C.c_void_p), ("ldy", C.c_int64), ("dy", C.c_void_p), ("lddy", C.c_int64),
+        ("mask", C.c_void_p), ("p", C.c_void_p), ("stream", C.c_void_p),
+    ]
+
+
 # every symbol include/megafold_amd.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "mf_version": (C.c_int, []),
@@ -76,6 +85,10 @@ SYMBOLS = {
     "mf_swiglu_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]),
     "mf_sigmoid_gate_fwd": (C.c_int, [C.POINTER(GateArgs)]),
     "mf_sigmoid_gate_bwd": (C.c_int, [C.POINTER(GateArgs)]),
+    "mf_trimul_pack_fwd": (C.c_int, [C.POINTER(TriMulArgs)]),
+    "mf_trimul_pack_bwd": (C.c_int, [C.POINTER(TriMulArgs)]),
+    "mf_channels_last_to_first": (C.c_int, [C.POINTER(TriMulArgs)]),
+    "mf_channels_first_to_last": (C.c_int, [C.POINTER(TriMulArgs)]),
 }
 
 _lock = threading.Lock()

@@ -73,17 +73,20 @@ def sigmoid_gate_forward(O2d: torch.Tensor, G: torch.Tensor) -> torch.Tensor:
     return A
 
 
-def sigmoid_gate_backward(dA: torch.Tensor, O2d: torch.Tensor, G: torch.Tensor, dG_out: torch.Tensor):
+def sigmoid_gate_backward(dA: torch.Tensor, O2d: torch.Tensor, G: torch.Tensor, dG_out: torch.Tensor,
+                          need_product: bool = True):
     """Returns ``(dO, A)`` and writes the gate gradient into ``dG_out`` (may be a column slice):
-    ``dO = dA * s``, ``dG = dA * O * s * (1 - s)``, ``A = O * s`` with ``s = sigmoid(G)``."""
+    ``dO = dA * s``, ``dG = dA * O * s * (1 - s)``, ``A = O * s`` with ``s = sigmoid(G)``; ``A`` is None
+    when ``need_product`` is false."""
     a = _gate_args(O2d, G)
     if dA.shape != O2d.shape or dA.dtype != O2d.dtype or dG_out.shape != O2d.shape or dG_out.dtype != O2d.dtype:
         raise ValueError("gate gradients must match the operands' shape and dtype")
     dA = dA if dA.stride(1) == 1 else dA.contiguous()
     with torch.cuda.device(O2d.device):
         dO = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device)
-        A = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device)
-        a.a, a.lda = A.data_ptr(), A.stride(0)
+        A = torch.empty(O2d.shape, dtype=O2d.dtype, device=O2d.device) if need_product else None
+        if A is not None:
+            a.a, a.lda = A.data_ptr(), A.stride(0)
         a.da, a.ldda = dA.data_ptr(), dA.stride(0)
         a.d_o, a.lddo = dO.data_ptr(), dO.stride(0)
         a.dg, a.lddg = dG_out.data_ptr(), dG_out.stride(0)

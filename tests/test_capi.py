@@ -215,3 +215,57 @@ def test_gate_struct_layout_matches_header(tmp_path):
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     a, b, c = map(int, subprocess.run([str(exe)], capture_output=True, text=True).stdout.split())
     assert (a, b, c) == (C.sizeof(_lib.GateArgs), _lib.GateArgs.da.offset, _lib.GateArgs.stream.offset)
+
+
+def _tm_args():
+    a = _lib.TriMulArgs()
+    a.B, a.n, a.np, a.dh, a.dtype = 1, 20, 24, 128, _lib.MF_BF16
+    a.y, a.dy, a.p = 0x10000, 0x20000, 0x30000           # never dereferenced: every check fails before a launch
+    a.ldy = a.lddy = 640
+    return a
+
+
+@pytest.mark.parametrize("mutate,code,text", [
+    (lambda a: setattr(a, "np", 20), -2, "multiple of 8"),
+    (lambda a: setattr(a, "np", 16), -2, ">= n"),
+    (lambda a: setattr(a, "n", 0), -2, "positive"),
+    (lambda a: setattr(a, "dh", 96), -2, "channels"),
+    (lambda a: setattr(a, "dtype", 7), -3, "dtype"),
+    (lambda a: setattr(a, "p", None), -1, "p is NULL"),
+    (lambda a: setattr(a, "y", None), -1, "y is NULL"),
+    (lambda a: setattr(a, "ldy", 500), -4, "y row stride"),
+    (lambda a: setattr(a, "y", 0x10002), -5, "y is not 16-byte aligned"),
+])
+def test_trimul_pack_argument_errors(mutate, code, text):
+    lib = _lib.lib()
+    a = _tm_args()
+    mutate(a)
+    assert lib.mf_trimul_pack_fwd(C.byref(a)) == code
+    assert text in lib.mf_last_error().decode()
+    assert lib.mf_trimul_pack_bwd(C.byref(a)) == code
+
+
+def test_channel_layout_argument_errors():
+    lib = _lib.lib()
+    a = _tm_args()
+    a.dh = 256                                            # plain forms move dh channels per row: 64, 128 or 256
+    a.ldy = a.lddy = 256
+    a.dy = None
+    assert lib.mf_channels_first_to_last(C.byref(a)) == -1 and "dy is NULL" in lib.mf_last_error().decode()
+    a = _tm_args()
+    a.dh = 32
+    assert lib.mf_channels_last_to_first(C.byref(a)) == -2 and "channels" in lib.mf_last_error().decode()
+    a = _tm_args()
+    a.lddy = 64
+    assert lib.mf_trimul_pack_bwd(C.byref(a)) == -4 and "dy row stride" in lib.mf_last_error().decode()
+    assert lib.mf_channels_last_to_first(None) == -1
+
+
+def test_trimul_struct_layout_matches_header(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include <stdio.h>\n#include "megafold_amd.h"\nint main(void){printf("%zu %zu %zu\\n", '
+                   'sizeof(mf_trimul_args), offsetof(mf_trimul_args, y), offsetof(mf_trimul_args, stream)); return 0;}\n')
+    exe = tmp_path / "t"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    a, b, c = map(int, subprocess.run([str(exe)], capture_output=True, text=True).stdout.split())
+    assert (a, b, c) == (C.sizeof(_lib.TriMulArgs), _lib.TriMulArgs.y.offset, _lib.TriMulArgs.stream.offset)
