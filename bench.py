@@ -156,22 +156,29 @@ def side_measurements(torch, steps, warmup):
     out["c5_bound_mib"] = 4 * 144 + 3 * 9
     del c5, q, k, v, bias, o
     torch.cuda.empty_cache()
-    out["triangle_attention_block"] = triangle_block(torch, steps, warmup)
+    out["triangle_attention_block"] = triangle_block(torch, steps, warmup, "attention")
+    out["triangle_multiplication_block"] = triangle_block(torch, steps, warmup, "multiplication")
     return out
 
 
-def triangle_block(torch, steps, warmup):
-    """fwd / bwd ms of the fused pre-LayerNorm triangle-attention block on a [1, 384, 384, 128] bf16 pair
-    tensor (heads 4 x 32, last 38 keys masked), both node types; autograd end to end, parameters in bf16."""
+def triangle_block(torch, steps, warmup, kind):
+    """fwd / bwd ms of the fused pair-stack blocks on a [1, 384, 384, 128] bf16 pair tensor with the last 38
+    positions masked: pre-LayerNorm triangle attention (heads 4 x 32, starting / ending node) or triangle
+    multiplication (outgoing / incoming); autograd end to end, parameters in bf16."""
     from megafold_amd.model.FusedTriangleAttention import PreLayerNormTriangleAttention
+    from megafold_amd.model.FusedTriangleMultiplication import TriangleMultiplication
     n, res = 384, {}
     g = torch.Generator().manual_seed(0)
     x = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda().requires_grad_()
     dout = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda()
     mask = torch.ones(1, n, dtype=torch.bool, device="cuda")
     mask[:, n - 38:] = False
-    for node_type in ("starting", "ending"):
-        m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type=node_type, dim_head=32).cuda().to(torch.bfloat16)
+    for node_type in (("starting", "ending") if kind == "attention" else ("outgoing", "incoming")):
+        if kind == "attention":
+            m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type=node_type, dim_head=32)
+        else:
+            m = TriangleMultiplication(dim=128, mix=node_type)
+        m = m.cuda().to(torch.bfloat16)
         with torch.no_grad():
             for p in m.parameters():
                 p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(p.dtype))
