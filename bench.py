@@ -158,6 +158,7 @@ def side_measurements(torch, steps, warmup):
     torch.cuda.empty_cache()
     out["triangle_attention_block"] = triangle_block(torch, steps, warmup, "attention")
     out["triangle_multiplication_block"] = triangle_block(torch, steps, warmup, "multiplication")
+    out["pairwise_block"] = triangle_block(torch, max(5, steps // 2), warmup, "pairwise")
     return out
 
 
@@ -167,17 +168,21 @@ def triangle_block(torch, steps, warmup, kind):
     multiplication (outgoing / incoming); autograd end to end, parameters in bf16."""
     from megafold_amd.model.FusedTriangleAttention import PreLayerNormTriangleAttention
     from megafold_amd.model.FusedTriangleMultiplication import TriangleMultiplication
+    from megafold_amd.model.PairwiseBlock import PairwiseBlock
     n, res = 384, {}
     g = torch.Generator().manual_seed(0)
     x = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda().requires_grad_()
     dout = torch.randn(1, n, n, 128, generator=g).to(torch.bfloat16).cuda()
     mask = torch.ones(1, n, dtype=torch.bool, device="cuda")
     mask[:, n - 38:] = False
-    for node_type in (("starting", "ending") if kind == "attention" else ("outgoing", "incoming")):
+    variants = {"attention": ("starting", "ending"), "multiplication": ("outgoing", "incoming"), "pairwise": ("all",)}
+    for node_type in variants[kind]:
         if kind == "attention":
             m = PreLayerNormTriangleAttention(dim=128, heads=4, node_type=node_type, dim_head=32)
-        else:
+        elif kind == "multiplication":
             m = TriangleMultiplication(dim=128, mix=node_type)
+        else:   # two multiplications, two attentions, transition, residual adds; dropout off
+            m = PairwiseBlock(dropout_row_prob=0.0, dropout_col_prob=0.0)
         m = m.cuda().to(torch.bfloat16)
         with torch.no_grad():
             for p in m.parameters():
@@ -186,7 +191,7 @@ def triangle_block(torch, steps, warmup, kind):
         for i in range(warmup + steps):       # no host synchronisation inside: launches stay ahead of the GPU
             e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
             e[0].record()
-            out = m(x, mask)
+            out = m(pairwise_repr=x, mask=mask) if kind == "pairwise" else m(x, mask)
             e[1].record()
             out.backward(dout)
             e[2].record()
@@ -199,6 +204,8 @@ def triangle_block(torch, steps, warmup, kind):
         tf = [e[0].elapsed_time(e[1]) for e in evs]
         tb = [e[1].elapsed_time(e[2]) for e in evs]
         res[node_type] = {"fwd_ms": round(median(tf), 4), "bwd_ms": round(median(tb), 4)}
+        del m, out
+        torch.cuda.empty_cache()
     return res
 
 

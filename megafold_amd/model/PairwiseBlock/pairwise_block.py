@@ -1,0 +1,52 @@
+"""The pair-stack block of the Pairformer / MSA module, assembled from the fused blocks (MI355X).
+
+Drop-in for ``PairwiseBlock`` of the reference (megafold/model/megafold.py:656-748): same constructor
+arguments, same sub-module names and therefore the same state-dict keys, same forward::
+
+    x = tri_mult_outgoing(x, mask) + x          megafold.py:742
+    x = tri_mult_incoming(x, mask) + x          megafold.py:743
+    x = tri_attn_starting(x, mask) + x          megafold.py:744
+    x = tri_attn_ending(x, mask) + x            megafold.py:745
+    x = pairwise_transition(x) + x              megafold.py:747
+
+Each of the five sub-blocks is one ``torch.autograd.Function`` over hand-written kernels; the residual adds
+are PyTorch's.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from ..FusedTransition.fused_transition import FusedTransition
+from ..FusedTriangleAttention.triangle_attention import PreLayerNormTriangleAttention
+from ..FusedTriangleMultiplication.triangle_multiplication import TriangleMultiplication
+
+__all__ = ["PairwiseBlock"]
+
+
+class PairwiseBlock(nn.Module):
+    def __init__(self, *, dim_pairwise=128, tri_mult_dim_hidden=None, tri_attn_dim_head=32, tri_attn_heads=4,
+                 dropout_row_prob=0.25, dropout_col_prob=0.25):
+        super().__init__()
+        tri_mult_kwargs = dict(dim=dim_pairwise, dim_hidden=tri_mult_dim_hidden)
+        tri_attn_kwargs = dict(dim=dim_pairwise, heads=tri_attn_heads, dim_head=tri_attn_dim_head)
+        self.tri_mult_outgoing = TriangleMultiplication(mix="outgoing", dropout=dropout_row_prob, dropout_type="row",
+                                                        **tri_mult_kwargs)
+        self.tri_mult_incoming = TriangleMultiplication(mix="incoming", dropout=dropout_row_prob, dropout_type="row",
+                                                        **tri_mult_kwargs)
+        self.tri_attn_starting = PreLayerNormTriangleAttention(node_type="starting", dropout=dropout_row_prob,
+                                                               dropout_type="row", **tri_attn_kwargs)
+        self.tri_attn_ending = PreLayerNormTriangleAttention(node_type="ending", dropout=dropout_col_prob,
+                                                             dropout_type="col", **tri_attn_kwargs)
+        self.pairwise_transition = FusedTransition(dim=dim_pairwise)
+
+    def forward(self, *, pairwise_repr: torch.Tensor, mask: Optional[torch.Tensor] = None, **kwargs) -> torch.Tensor:
+        x = pairwise_repr
+        x = self.tri_mult_outgoing(x, mask=mask) + x
+        x = self.tri_mult_incoming(x, mask=mask) + x
+        x = self.tri_attn_starting(x, mask=mask) + x
+        x = self.tri_attn_ending(x, mask=mask) + x
+        x = self.pairwise_transition(x) + x
+        return x

@@ -1,0 +1,71 @@
+"""PairwiseBlock assembled from the fused blocks: parameter names against the reference's state-dict keys
+(CPU), and parity of output, input gradient and every parameter gradient against the composed oracle (GPU)."""
+import pytest
+import torch
+
+from megafold_amd.model.PairwiseBlock import PairwiseBlock
+from oracle import pairwise_block as opb
+
+# state-dict keys of PairwiseBlock() in the reference (megafold/model/megafold.py:659-723 with the sub-modules'
+# own parameters: TriangleMultiplication :441-458, PreLayerNorm :318-319, TriangleAttention :609-615, Attention
+# attention.py:135-158, FusedTransition FusedTransition/fused_transition.py:128-131)
+TM = ["combined.WEIGHT", "combined.BIAS", "combined.linear_weight", "combined.linear_bias",
+      "to_out.0.WEIGHT", "to_out.0.BIAS", "to_out.0.linear_weight"]
+TA = ["norm.weight", "norm.bias", "fn.to_attn_bias.0.weight", "fn.attn.to_q.weight", "fn.attn.to_q.bias",
+      "fn.attn.to_kv.weight", "fn.attn.to_out.weight", "fn.attn.to_gates.weight", "fn.attn.to_gates.bias"]
+TR = ["ff.0.WEIGHT", "ff.0.BIAS", "ff.0.linear_weight", "ff.2.weight"]
+REFERENCE_KEYS = ({"tri_mult_outgoing." + k for k in TM} | {"tri_mult_incoming." + k for k in TM} |
+                  {"tri_attn_starting." + k for k in TA} | {"tri_attn_ending." + k for k in TA} |
+                  {"pairwise_transition." + k for k in TR})
+
+
+def test_parameter_names_match_the_reference():
+    m = PairwiseBlock()
+    assert set(m.state_dict().keys()) == REFERENCE_KEYS
+    assert m.tri_attn_ending.fn.dropout.dropout_type == "col" and m.tri_mult_incoming.to_out[1].dropout_type == "row"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,masked,dtype", [(40, 4, torch.bfloat16), (24, 0, torch.float32)])
+def test_block_parity(n, masked, dtype):
+    from conftest import tol_for
+    torch.manual_seed(n)
+    m = PairwiseBlock(dropout_row_prob=0.0, dropout_col_prob=0.0)
+    g = torch.Generator().manual_seed(n + 1)
+    with torch.no_grad():
+        for name, p in m.named_parameters():
+            if name.endswith(("WEIGHT", "norm.weight")):
+                p.copy_(1 + 0.1 * torch.randn(p.shape, generator=g))
+            elif p.dim() == 1:
+                p.copy_(0.1 * torch.randn(p.shape, generator=g))
+            else:
+                fan_in = p.shape[0] if name.endswith("linear_weight") else p.shape[1]
+                p.copy_(torch.randn(p.shape, generator=g) * fan_in ** -0.5)
+    m = m.to(dtype)
+    x = torch.randn(1, n, n, 128, generator=g).to(dtype)
+    dout = torch.randn(1, n, n, 128, generator=g).to(dtype)
+    mask = None
+    if masked:
+        mask = torch.ones(1, n, dtype=torch.bool)
+        mask[:, n - masked:] = False
+    params = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    want_out, want_dx, want_dp = opb.pairwise_block_forward_backward(x, mask, params, dout, 4, 32)
+
+    m = m.cuda()
+    xg = x.cuda().requires_grad_(True)
+    out = m(pairwise_repr=xg, mask=mask.cuda() if mask is not None else None)
+    out.backward(dout.cuda())
+    tol = tol_for(dtype)
+    if dtype != torch.float32:
+        tol = dict(rtol=4e-2, atol=4e-2)     # five 16-bit blocks in sequence: twice the single-block bar
+
+    def close(name, got, want):
+        assert not torch.isnan(got).any(), name
+        got = got.detach().cpu().double()
+        s = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(got / s, want / s, msg=lambda msg: "%s: %s" % (name, msg), **tol)
+
+    close("out", out, want_out)
+    close("dx", xg.grad, want_dx)
+    for name, p in m.named_parameters():
+        close(name, p.grad, want_dp[name])
