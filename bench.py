@@ -141,7 +141,28 @@ def side_measurements(torch, steps, warmup):
                            "bwd_GBps": round(bb / tb / 1e6, 1), "fwd_frac_hbm": round(bf / tf / 1e6 / PEAK_HBM_GBS, 4),
                            "bwd_frac_hbm": round(bb / tb / 1e6 / PEAK_HBM_GBS, 4),
                            "fwd_TFLOPs": round(2.0 * M * K * N1 / tf / 1e9, 1)}
-    del h, x2, Mean, RSTD, dh, tin, inp
+    # the whole FusedTransition module (adds the output projection and its gradients, BLAS)
+    from megafold_amd.model.FusedTransition.fused_transition import FusedTransition
+    mod = FusedTransition(128, 4, device="cuda", dtype=torch.bfloat16)
+    xm = tin["x"].clone().requires_grad_()
+    dym = torch.randn_like(tin["x"])
+    evs = []
+    for i in range(warmup + steps):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record()
+        ym = mod(xm)
+        e[1].record()
+        ym.backward(dym)
+        e[2].record()
+        xm.grad = None
+        for p_ in mod.parameters():
+            p_.grad = None
+        if i >= warmup:
+            evs.append(e)
+    torch.cuda.synchronize()
+    out["transition_module_c4"] = {"fwd_ms": round(median([e[0].elapsed_time(e[1]) for e in evs]), 4),
+                                   "bwd_ms": round(median([e[1].elapsed_time(e[2]) for e in evs]), 4)}
+    del h, x2, Mean, RSTD, dh, tin, inp, mod, xm, dym, ym
     torch.cuda.empty_cache()
     c5 = {k: v.cuda() for k, v in workloads.config5().items()}
     q, k, v = (c5[n].requires_grad_() for n in "qkv")

@@ -19,6 +19,7 @@ import torch.nn as nn
 
 from ... import _lib
 from ..FusedLayernormLinear.fused_layernorm_linear import LayernormLinear
+from ..linear import linear_no_bias
 
 __all__ = ["FusedTransition", "FusedSwiGLU", "FusedSwiGLUFunction", "swiglu_forward", "swiglu_backward"]
 
@@ -119,10 +120,15 @@ class FusedTransition(nn.Module):
             )
 
     def forward(self, input):
+        # the output projection (ff[-1], a bias-free nn.Linear) runs through linear_no_bias: same GEMMs,
+        # but a weight gradient that is split along the long row axis
         if self._fused_ln_swiglu:
             # LayerNorm -> Linear -> SwiGLU in one kernel, then the output projection
-            return self.ff[2](self.ff[0](input, act=_lib.MF_ACT_SWIGLU))
-        return self.ff(input)
+            return linear_no_bias(self.ff[0](input, act=_lib.MF_ACT_SWIGLU), self.ff[2].weight)
+        h = input
+        for layer in list(self.ff)[:-1]:
+            h = layer(h)
+        return linear_no_bias(h, self.ff[-1].weight)
 
     def extra_repr(self):
         return f"dim={self.dim}, dim_inner={self.dim_inner}"

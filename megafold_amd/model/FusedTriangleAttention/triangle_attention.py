@@ -41,6 +41,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ... import _lib
+from ..linear import tall_skinny_tn
 from ..FusedEvoAttention.evoattention import evoattention_backward, evoattention_forward
 from ..FusedLayernormLinear.fused_layernorm_linear import (fused_shape_supported, layernorm_linear_backward,
                                                            layernorm_linear_forward)
@@ -92,22 +93,6 @@ def sigmoid_gate_backward(dA: torch.Tensor, O2d: torch.Tensor, G: torch.Tensor, 
         a.dg, a.lddg = dG_out.data_ptr(), dG_out.stride(0)
         _lib.check(_lib.lib().mf_sigmoid_gate_bwd(C.byref(a)), "mf_sigmoid_gate_bwd")
     return dO, A
-
-
-def _tall_skinny_tn(X: torch.Tensor, Y: torch.Tensor) -> torch.Tensor:
-    """``X^T Y`` for X ``[M, p]``, Y ``[M, q]`` with M much larger than p, q (a weight gradient): the long
-    axis is split into slices that run as one batched GEMM and are then summed in fp32, which fills the
-    device where a single [p, M] x [M, q] product would run on a handful of work-groups."""
-    M = X.shape[0]
-    split = 1
-    for cand in (256, 128, 64, 32, 16, 8, 4, 2):
-        if M % cand == 0 and M // cand >= 256:
-            split = cand
-            break
-    if split == 1:
-        return X.t() @ Y
-    part = torch.bmm(X.view(split, M // split, X.shape[1]).transpose(1, 2), Y.view(split, M // split, Y.shape[1]))
-    return part.sum(0, dtype=torch.float32).to(X.dtype)
 
 
 def _views(Y: torch.Tensor, b: int, n: int, heads: int, dh: int):
@@ -172,7 +157,7 @@ class TriangleAttentionFunction(torch.autograd.Function):
         dY = torch.empty_like(Y)
         dQ, dK, dV, dG, dBv = _views(dY, b, n, heads, dh)
         dO, A = sigmoid_gate_backward(dA, O2d, G, dG)
-        dWo = _tall_skinny_tn(dout2d, A)                  # [d, inner]
+        dWo = tall_skinny_tn(dout2d, A)                  # [d, inner]
         dO = dO.view(b, n, n, heads, dh)
         _, _, _, dbias = evoattention_backward(dO, Q, K, V, mask5, Bv, O, lse, True, out=(dQ, dK, dV))
         dY.as_strided((b, heads, n, n), (n * n * Nt, 1, n * Nt, Nt), dY.storage_offset() + 4 * inner).copy_(dbias[:, 0])

@@ -1,0 +1,55 @@
+"""Plain (bias-free) linear layers of the fused blocks: BLAS GEMMs with a weight gradient that fills the device.
+
+The output projections of the pair stack multiply ``[M, in]`` activations with M = b * n * n rows (147456 at
+n = 384) by small ``[out, in]`` weights (``nn.Linear(dim_inner, dim, bias=False)`` of the transition,
+megafold/model/FusedTransition/fused_transition.py:130; ``to_out`` of the attention,
+megafold/model/attention.py:133).  Their weight gradient ``dY^T X`` is a ``[out, M] x [M, in]`` product whose
+long axis is the contraction: as ONE GEMM the BLAS library runs it on a handful of work-groups (425 us for
+128 x 147456 x 512 in bf16).  Here the long axis is split into slices that run as one batched GEMM and are
+summed in fp32 (about 30 us).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+__all__ = ["tall_skinny_tn", "LinearNoBiasFunction", "linear_no_bias"]
+
+
+def tall_skinny_tn(X: torch.Tensor, Y: torch.Tensor) -> torch.Tensor:
+    """``X^T Y`` for X ``[M, p]``, Y ``[M, q]`` with M much larger than p and q."""
+    M = X.shape[0]
+    split = 1
+    for cand in (256, 128, 64, 32, 16, 8, 4, 2):
+        if M % cand == 0 and M // cand >= 256:
+            split = cand
+            break
+    if split == 1:
+        return X.t() @ Y
+    part = torch.bmm(X.view(split, M // split, X.shape[1]).transpose(1, 2), Y.view(split, M // split, Y.shape[1]))
+    return part.sum(0, dtype=torch.float32).to(X.dtype)
+
+
+class LinearNoBiasFunction(torch.autograd.Function):
+    """``x @ weight^T`` with ``weight [out, in]`` as ``nn.Linear`` stores it."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx, x, weight):
+        w = weight if weight.dtype == x.dtype else weight.to(x.dtype)
+        ctx.save_for_backward(x, w)
+        return F.linear(x, w)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        dy2 = dy2 if dy2.dtype == x.dtype else dy2.to(x.dtype)
+        dx = (dy2 @ w).view(x.shape) if ctx.needs_input_grad[0] else None
+        dw = tall_skinny_tn(dy2.contiguous(), x.reshape(-1, x.shape[-1])) if ctx.needs_input_grad[1] else None
+        return dx, dw
+
+
+def linear_no_bias(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    return LinearNoBiasFunction.apply(x, weight)
