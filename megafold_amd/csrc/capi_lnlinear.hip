@@ -31,7 +31,7 @@ LnPlan make_plan(const mf_lnlinear_args* a, bool backward) {
     pl.off_bp = off; off += align256((uint64_t)a->N * 4);
   }
   if (backward) {
-    pl.R = ln_row_ranges(a->M, a->N);
+    pl.R = ln_row_ranges(a->M, a->K, a->N);
     pl.rows_per_range = (a->M + pl.R - 1) / pl.R;
     pl.off_wg = off; off += align256((uint64_t)a->K * a->N * es);
     pl.off_g = off; off += align256((uint64_t)pl.R * a->K * a->N * 4);

@@ -58,6 +58,6 @@ hipError_t launch_swiglu_fwd(const void* x, void* y, int64_t M, int Dh, int dtyp
 hipError_t launch_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t M, int Dh, int dtype, hipStream_t stream);
 
 int ln_padded_k(int K);                 // padded K of the kernels, 0 if K is unsupported
-int ln_row_ranges(int64_t M, int N);    // R for the weight-gradient partials
+int ln_row_ranges(int64_t M, int K, int N);    // R for the weight-gradient partials
 
 }  // namespace mf

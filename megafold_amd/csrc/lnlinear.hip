@@ -113,11 +113,17 @@ int ln_padded_k(int K) {
   return 0;
 }
 
-int ln_row_ranges(int64_t M, int N) {
-  // about two work-groups per compute unit over (ranges x column blocks); each range at least 256 rows
-  int64_t r = 128;
-  while (r > 1 && M / r < 256) r /= 2;
-  (void)N;
+int ln_row_ranges(int64_t M, int K, int N) {
+  // The weight-gradient kernel runs (ranges x column blocks) work-groups, two resident per compute unit:
+  // the number of ranges is chosen so that the grid is ONE round of resident work-groups (a grid of 1.25
+  // rounds costs two), with at least 256 rows per range.
+  const int KP = ln_padded_k(K);
+  const int cw = KP > 128 ? 64 : 128;                    // columns per work-group (DwShape<KP>::CW)
+  const int gy = (N + cw - 1) / cw;
+  int64_t r = 2LL * num_cu() / (gy > 0 ? gy : 1);
+  if (r > M / 256) r = M / 256;
+  if (r > 1024) r = 1024;
+  if (r < 1) r = 1;
   return (int)r;
 }
 
