@@ -788,8 +788,13 @@ hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream) {
 // =================================================================================================
 // dBias
 // =================================================================================================
-template <typename T, int DP, int TR>
-__global__ void __launch_bounds__(256, (sizeof(T) == 4 && DP > 32) ? 1 : 2)
+// HP = heads per work-group.  With H * D 16-bit values per position two neighbouring heads share every
+// 128-byte line of Q, K, V and dO, and the L1 fetches whole lines: a work-group that handles one head
+// moves twice the bytes it uses (this kernel is bound by exactly that L2 -> L1 stream).  With HP = 2 the
+// work-group has eight wavefronts, four per head of a pair, working on the same patch and row in step, so
+// the second head finds its half of every line in the L1.
+template <typename T, int DP, int TR, int HP>
+__global__ void __launch_bounds__(256 * HP, HP == 2 ? 1 : ((sizeof(T) == 4 && DP > 32) ? 1 : 2))
 evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   constexpr int AHEAD = DP <= 32 ? 2 : 1;
   using L = BwdLayout<T, DP>;
@@ -799,31 +804,55 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   constexpr int ITEMS = ROWS * CPR;
   constexpr int PF = (ITEMS + 255) / 256;
 
+  const int tid = threadIdx.x & 255, hs = threadIdx.x >> 8;      // hs: head inside the pair (HP = 2)
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T* Ks = reinterpret_cast<T*>(smem_raw);       // [2][ROWS][KSTR]
-  T* Vs = Ks + 2 * ROWS * L::KSTR;              // [2][ROWS][QSTR]
+  // per head: K [2][ROWS][KSTR], V [2][ROWS][QSTR] and, with HP = 2, the query-side tiles Q, dO [2][128][QSTR]
+  constexpr int QT_ELEMS = HP == 2 ? 2 * 128 * L::QSTR : 0;
+  constexpr int HEAD_ELEMS = 2 * ROWS * (L::KSTR + L::QSTR) + 2 * QT_ELEMS;
+  T* const lds0 = reinterpret_cast<T*>(smem_raw);
+  T* Ks = lds0 + hs * HEAD_ELEMS;
+  T* Vs = Ks + 2 * ROWS * L::KSTR;
+  T* Qs = Vs + 2 * ROWS * L::QSTR;              // HP = 2 only
+  T* dOs = Qs + QT_ELEMS;
 
   const int R = IB * JB;
-  const int G = p.B * p.H * p.n_chunks;
   const int bid = blockIdx.x;
   const int xcd = bid & 7, kq = bid >> 3;
-  // Each XCD takes a contiguous run of groups (b, head pair, chunk, head in pair): with H * D 16-bit
-  // values per (row, position) two neighbouring heads share every 128-byte line of Q, K, V and dO, so
-  // they should meet in one L2 (otherwise each XCD fetches the line for half of its bytes).  With an
-  // odd run length some pairs straddle two XCDs; the run length is what balances the device.
-  const int hp = (p.H & 1) ? 1 : 2;
-  const int gpx = (G + 7) / 8;                             // groups per XCD
-  const int grp = xcd * gpx + kq / R;
-  if (grp >= G) return;
-  const int reg = kq % R;
+  int h, b, chunk, reg;
+  if (HP == 2) {
+    // (b, head pair, chunk) groups of R patches, dealt out evenly: XCD x takes the contiguous run
+    // [x * per_xcd, (x + 1) * per_xcd) of the (group, patch) list, so that a group's patches (which share
+    // Q, K, V, dO) stay in at most two L2s while every XCD gets the same number of work-groups
+    const int64_t total = (int64_t)p.B * (p.H / 2) * p.n_chunks * R;
+    const int64_t per_xcd = (total + 7) / 8;
+    const int64_t q = xcd * per_xcd + kq;
+    if (kq >= per_xcd || q >= total) return;
+    const int grp = (int)(q / R);
+    reg = (int)(q % R);
+    chunk = grp % p.n_chunks;
+    const int hb = grp / p.n_chunks;
+    h = (hb % (p.H / 2)) * 2 + hs;
+    b = hb / (p.H / 2);
+  } else {
+    const int G = p.B * p.H * p.n_chunks;
+    // Each XCD takes a contiguous run of groups (b, head pair, chunk, head in pair): the two heads of a
+    // pair share every 128-byte line, so they should at least meet in one L2.  With an odd run length
+    // some pairs straddle two XCDs; the run length is what balances the device.
+    const int hp = (p.H & 1) ? 1 : 2;
+    const int gpx = (G + 7) / 8;                             // groups per XCD
+    const int grp = xcd * gpx + kq / R;
+    if (grp >= G) return;
+    reg = kq % R;
+    // grp = ((b * (H / hp) + head pair) * n_chunks + chunk) * hp + head inside the pair
+    const int hsub = grp % hp;
+    chunk = (grp / hp) % p.n_chunks;
+    const int hb = grp / hp / p.n_chunks;
+    h = (hb % (p.H / hp)) * hp + hsub;
+    b = hb / (p.H / hp);
+  }
   const int ib = reg % IB, jb = reg / IB;
-  // grp = ((b * (H / hp) + head pair) * n_chunks + chunk) * hp + head inside the pair
-  const int hsub = grp % hp;
-  const int chunk = (grp / hp) % p.n_chunks;
-  const int hb = grp / hp / p.n_chunks;
-  const int h = (hb % (p.H / hp)) * hp + hsub, b = hb / (p.H / hp);
 
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
+  const int w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int S = p.S, D = p.D;
   const int n_begin = chunk * p.rows_per_chunk;
   const int n_end = min(p.N, n_begin + p.rows_per_chunk);
@@ -837,6 +866,15 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   const T* Kg = reinterpret_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
   const T* Vg = reinterpret_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
   const float* biasg = p.bias + b * p.bias_sb + h * p.bias_sh;
+  // HP = 2: the eight wavefronts stage both heads together, one whole 128-byte line (2 heads x 32 values)
+  // per eight lanes, so the pointers below address head 2 * pair; the launcher has checked that the head
+  // stride of Q, K, V, dO is D = 32 elements.
+  const int t512 = threadIdx.x;
+  const int c8 = t512 & 7;                               // 16-byte chunk of the pair line: head c8 >> 2, chunk c8 & 3
+  const T* Kp = reinterpret_cast<const T*>(p.k.ptr) + b * p.k.sb + (h - hs) * p.k.sh + 8 * c8;
+  const T* Vp = reinterpret_cast<const T*>(p.v.ptr) + b * p.v.sb + (h - hs) * p.v.sh + 8 * c8;
+  const T* Qp = reinterpret_cast<const T*>(p.q.ptr) + b * p.q.sb + (h - hs) * p.q.sh + 8 * c8;
+  const T* dOp = reinterpret_cast<const T*>(p.dO.ptr) + b * p.dO.sb + (h - hs) * p.dO.sh + 8 * c8;
 
   const float cexp = p.scale * MF_LOG2E;   // the accumulator holds z / scale
   const float inv_scale = 1.0f / p.scale;
@@ -872,17 +910,24 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   const int mask_es = p.mask_dtype == MF_F32 ? 4 : (p.mask_dtype == MF_F16 || p.mask_dtype == MF_BF16) ? 2 : 1;
   const int mj = jt0 * 32 + tid < S ? jt0 * 32 + tid : S - 1;     // mask column of the threads tid < ROWS
   auto fetch = [&](int n, Staged& st) {
-    const T* kn = Kg + (int64_t)n * p.k.sn;
-    const T* vn = Vg + (int64_t)n * p.v.sn;
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int c = tid + 256 * i;
-      const int kk = (c < ITEMS ? c : 0) / CPR, dc = c % CPR;
-      int j = jt0 * 32 + kk;
+    if constexpr (HP == 2) {
+      int j = jt0 * 32 + (t512 >> 3);                    // 64 key rows x 8 chunks = 512 threads
       j = j < S ? j : S - 1;
-      const int d0 = 8 * dc < D ? 8 * dc : 0;
-      st.k[i] = ld8<T>(kn + (int64_t)j * p.k.ss + d0);
-      st.v[i] = ld8<T>(vn + (int64_t)j * p.v.ss + d0);
+      st.k[0] = ld8<T>(Kp + (int64_t)n * p.k.sn + (int64_t)j * p.k.ss);
+      st.v[0] = ld8<T>(Vp + (int64_t)n * p.v.sn + (int64_t)j * p.v.ss);
+    } else {
+      const T* kn = Kg + (int64_t)n * p.k.sn;
+      const T* vn = Vg + (int64_t)n * p.v.sn;
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+        const int c = tid + 256 * i;
+        const int kk = (c < ITEMS ? c : 0) / CPR, dc = c % CPR;
+        int j = jt0 * 32 + kk;
+        j = j < S ? j : S - 1;
+        const int d0 = 8 * dc < D ? 8 * dc : 0;
+        st.k[i] = ld8<T>(kn + (int64_t)j * p.k.ss + d0);
+        st.v[i] = ld8<T>(vn + (int64_t)j * p.v.ss + d0);
+      }
     }
     {
       const unsigned char* mp = reinterpret_cast<const unsigned char*>(p.mask) +
@@ -891,12 +936,22 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
       else if (mask_es == 2) st.mraw = *reinterpret_cast<const unsigned short*>(mp);
       else st.mraw = *mp;
     }
+    if constexpr (HP == 2) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int d0 = (DP / 2) * g + 8 * s;
-      const int dcl = d0 < D ? d0 : 0;
-      st.q[s] = ld8<T>(Qg + (int64_t)n * p.q.sn + dcl);
-      st.dO[s] = ld8<T>(dOg + (int64_t)n * p.dO.sn + dcl);
+      for (int i = 0; i < 2; ++i) {                      // 128 query rows x 8 chunks = 2 x 512 threads
+        int qr = ib * 128 + 64 * i + (t512 >> 3);
+        qr = qr < S ? qr : S - 1;
+        st.q[i] = ld8<T>(Qp + (int64_t)n * p.q.sn + (int64_t)qr * p.q.ss);
+        st.dO[i] = ld8<T>(dOp + (int64_t)n * p.dO.sn + (int64_t)qr * p.dO.ss);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int d0 = (DP / 2) * g + 8 * s;
+        const int dcl = d0 < D ? d0 : 0;
+        st.q[s] = ld8<T>(Qg + (int64_t)n * p.q.sn + dcl);
+        st.dO[s] = ld8<T>(dOg + (int64_t)n * p.dO.sn + dcl);
+      }
     }
     const int64_t ridx = (((int64_t)b * p.N + n) * p.H + h) * S + qi_c;
     st.lraw = p.lse[ridx];
@@ -905,15 +960,36 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   auto stash = [&](int buf, const Staged& st) {
     T* kd = Ks + buf * ROWS * L::KSTR;
     T* vd = Vs + buf * ROWS * L::QSTR;
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int c = tid + 256 * i;
-      if (c < ITEMS) {
-        const int kk = c / CPR, dc = c % CPR;
+    if constexpr (HP == 2) {
+      // this thread's chunk belongs to head c8 >> 2: write it into that head's tiles
+      T* const hb = lds0 + (c8 >> 2) * HEAD_ELEMS;
+      const int dc = c8 & 3;
+      {
+        const int kk = t512 >> 3;
         const int row = (kk & ~31) + perm32(kk & 31);
-        const bool ok = jt0 * 32 + kk < S && 8 * dc < D;
-        st8<T>(kd + row * L::KSTR + 8 * dc, ok ? st.k[i] : frag_zero<T>());
-        st8<T>(vd + row * L::QSTR + 8 * dc, ok ? st.v[i] : frag_zero<T>());
+        const bool ok = jt0 * 32 + kk < S;
+        st8<T>(hb + (buf * ROWS + row) * L::KSTR + 8 * dc, ok ? st.k[0] : frag_zero<T>());
+        st8<T>(hb + 2 * ROWS * L::KSTR + (buf * ROWS + row) * L::QSTR + 8 * dc, ok ? st.v[0] : frag_zero<T>());
+      }
+      T* const qb = hb + 2 * ROWS * (L::KSTR + L::QSTR) + buf * 128 * L::QSTR;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = 64 * i + (t512 >> 3);
+        const bool ok = ib * 128 + row < S;
+        st8<T>(qb + row * L::QSTR + 8 * dc, ok ? st.q[i] : frag_zero<T>());
+        st8<T>(qb + QT_ELEMS + row * L::QSTR + 8 * dc, ok ? st.dO[i] : frag_zero<T>());
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+        const int c = tid + 256 * i;
+        if (c < ITEMS) {
+          const int kk = c / CPR, dc = c % CPR;
+          const int row = (kk & ~31) + perm32(kk & 31);
+          const bool ok = jt0 * 32 + kk < S && 8 * dc < D;
+          st8<T>(kd + row * L::KSTR + 8 * dc, ok ? st.k[i] : frag_zero<T>());
+          st8<T>(vd + row * L::QSTR + 8 * dc, ok ? st.v[i] : frag_zero<T>());
+        }
       }
     }
     if (tid < ROWS) {
@@ -936,20 +1012,33 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   // one row n: consume the staged set, publish K / V, request row n + AHEAD into the same set, compute
   auto row_step = [&](int n, int buf, Staged& st) {
     frag qc[KS], doc[KS];
+    if constexpr (HP != 2) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const bool ok = qi < S && (DP / 2) * g + 8 * s < D;
-      qc[s] = ok ? st.q[s] : frag_zero<T>();
-      doc[s] = ok ? st.dO[s] : frag_zero<T>();
+      for (int s = 0; s < KS; ++s) {
+        const bool ok = qi < S && (DP / 2) * g + 8 * s < D;
+        qc[s] = ok ? st.q[s] : frag_zero<T>();
+        doc[s] = ok ? st.dO[s] : frag_zero<T>();
+      }
     }
     float l2p = (qi < S && st.lraw != -__builtin_inff()) ? st.lraw * MF_LOG2E : __builtin_inff();
     float dlc = st.draw;
+    if constexpr (HP != 2) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) { pin(qc[s]); pin(doc[s]); }
+      for (int s = 0; s < KS; ++s) { pin(qc[s]); pin(doc[s]); }
+    }
     pin(l2p); pin(dlc);
     stash(buf, st);
     __syncthreads();
     fetch(n + AHEAD < n_end ? n + AHEAD : n_end - 1, st);   // the tail repeats the last row rather than branching around loads
+    if constexpr (HP == 2) {
+      // this lane's query row of its own head, staged by the whole work-group
+      const T* qrow = Qs + (buf * 128 + w * 32 + x) * L::QSTR + (DP / 2) * g;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        qc[s] = ld8<T>(qrow + 8 * s);
+        doc[s] = ld8<T>(qrow + QT_ELEMS + 8 * s);
+      }
+    }
 
     const T* kt = Ks + buf * ROWS * L::KSTR;
     const T* vt = Vs + buf * ROWS * L::QSTR;
@@ -1062,41 +1151,49 @@ static int dbias_num_cu() {
 // ceil(N / chunks) row steps.  Every chunk also costs one partial [B, H, S, S] buffer that is written
 // and read back, priced in row steps (about 1.4 us) at about 2 TB/s so that near-ties go to the
 // smaller workspace.  Pick the chunk count with the smallest estimate.
+// Two heads per work-group (see the kernel) for the 16-bit types at D <= 32 when the heads pair up.
+static bool dbias_pairs_heads(int dtype, int D, int H) { return dtype != MF_F32 && D <= 32 && (H & 1) == 0; }
+
 int evo_dbias_chunks(int B, int N, int S, int H, int D, int dtype) {
   const int TR = dbias_tr(dtype, D);
   const int NT = (S + 31) / 32;
   const int IB = (S + 127) / 128, JB = (NT + TR - 1) / TR;
   const long long regions = (long long)IB * JB;
-  const long long slots_xcd = 2LL * (dbias_num_cu() / 8 > 0 ? dbias_num_cu() / 8 : 1);
+  const bool pairs = dbias_pairs_heads(dtype, D, H);
+  const long long cu_xcd = dbias_num_cu() / 8 > 0 ? dbias_num_cu() / 8 : 1;
+  const long long slots_xcd = pairs ? cu_xcd : 2 * cu_xcd;          // eight-wavefront groups: one per compute unit
   const double part_cost = (double)B * H * S * S * 8.0 / 2.0e12 / 1.4e-6;
   int best = 1;
   double best_cost = -1.0;
   for (int c = 1; c <= 8 && c <= N; ++c) {     // at most 8 partial buffers: they count as activation memory
     const int rows = (N + c - 1) / c;
     if ((N + rows - 1) / rows != c) continue;
-    const long long groups_xcd = ((long long)B * H * c + 7) / 8;
-    const long long rounds = (groups_xcd * regions + slots_xcd - 1) / slots_xcd;
+    // work-groups of the busiest XCD: whole groups per XCD, or (paired heads) an even split of all patches
+    const long long wg_xcd = pairs ? ((long long)B * (H / 2) * c * regions + 7) / 8
+                                   : (((long long)B * H * c + 7) / 8) * regions;
+    const long long rounds = (wg_xcd + slots_xcd - 1) / slots_xcd;
     const double cost = (double)rounds * rows + (c > 1 ? c * part_cost : 0.0);
     if (best_cost < 0.0 || cost < best_cost) { best_cost = cost; best = c; }
   }
   return best;
 }
 
-template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const EvoParams& p, hipStream_t stream) {
+template <typename T, int DP, int TR, int HP> static hipError_t launch_dbias_t(const EvoParams& p, hipStream_t stream) {
   using L = BwdLayout<T, DP>;
   const int NT = (p.S + 31) / 32;
   const int IB = (p.S + 127) / 128, JB = (NT + TR - 1) / TR;
-  const size_t smem = (size_t)2 * TR * 32 * (L::KSTR + L::QSTR) * sizeof(T);
-  const long long G = (long long)p.B * p.H * p.n_chunks;
-  const long long blocks = (G + 7) / 8 * 8 * IB * JB;
+  const size_t smem = (size_t)HP * (2 * TR * 32 * (L::KSTR + L::QSTR) + (HP == 2 ? 4 * 128 * L::QSTR : 0)) * sizeof(T);
+  long long blocks;
+  if (HP == 2) blocks = ((long long)p.B * (p.H / 2) * p.n_chunks * IB * JB + 7) / 8 * 8;
+  else blocks = ((long long)p.B * p.H * p.n_chunks + 7) / 8 * 8 * IB * JB;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kern = evo_bwd_dbias_kernel<T, DP, TR>;
+  auto kern = evo_bwd_dbias_kernel<T, DP, TR, HP>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, stream, p, IB, JB);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256 * HP), smem, stream, p, IB, JB);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (p.n_chunks > 1) {
@@ -1113,8 +1210,14 @@ template <typename T, int DP, int TR> static hipError_t launch_dbias_t(const Evo
 
 template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipStream_t stream) {
   constexpr bool wide = sizeof(T) == 4;
-  if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 2>(p, stream);
-  if (p.D <= 64) return launch_dbias_t<T, 64, 1>(p, stream);
+  if constexpr (!wide) {
+    // whole-line staging of a head pair needs the two heads side by side in memory (D = 32 exactly)
+    if (dbias_pairs_heads(p.dtype, p.D, p.H) && p.D == 32 && p.q.sh == 32 && p.k.sh == 32 && p.v.sh == 32 &&
+        p.dO.sh == 32)
+      return launch_dbias_t<T, 32, 2, 2>(p, stream);
+  }
+  if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 2, 1>(p, stream);
+  if (p.D <= 64) return launch_dbias_t<T, 64, 1, 1>(p, stream);
   return hipErrorInvalidValue;
 }
 
