@@ -71,3 +71,48 @@ def transition_inputs(M_shape=(1, 384, 384), dim=128, expansion_factor=4, dtype=
     W2 = (_randn(gen, dim, di) / math.sqrt(di)).to(dtype)
     dY = _randn(gen, *M_shape, dim).to(dtype)
     return {"x": x, "gamma": gamma, "beta": beta, "W1": W1, "W2": W2, "dY": dY}
+
+
+def _pair_mask(b, n, n_masked):
+    if not n_masked:
+        return None
+    mask = torch.ones(b, n, dtype=torch.bool)
+    mask[:, n - n_masked:] = False
+    return mask
+
+
+def triangle_attention_inputs(b=1, n=12, dim=64, heads=2, dim_head=16, n_masked=3, dtype=torch.float32, seed=0):
+    """Pair tensor ``[b, n, n, dim]``, key mask ``[b, n]`` (last ``n_masked`` positions off), upstream gradient and
+    the parameters of ``PreLayerNorm(TriangleAttention)`` under the reference's state-dict names.
+    Draw order: x, dout, then the parameters in the order of the dict."""
+    gen = torch.Generator().manual_seed(seed)
+    inner = heads * dim_head
+    x = _randn(gen, b, n, n, dim).to(dtype)
+    dout = _randn(gen, b, n, n, dim).to(dtype)
+    params = {
+        "norm.weight": 1 + 0.1 * _randn(gen, dim), "norm.bias": 0.1 * _randn(gen, dim),
+        "fn.to_attn_bias.0.weight": _randn(gen, heads, dim) * dim ** -0.5,
+        "fn.attn.to_q.weight": _randn(gen, inner, dim) * dim ** -0.5, "fn.attn.to_q.bias": 0.1 * _randn(gen, inner),
+        "fn.attn.to_kv.weight": _randn(gen, 2 * inner, dim) * dim ** -0.5,
+        "fn.attn.to_out.weight": _randn(gen, dim, inner) * inner ** -0.5,
+        "fn.attn.to_gates.weight": _randn(gen, inner, dim) * dim ** -0.5,
+        "fn.attn.to_gates.bias": 0.1 * _randn(gen, inner) - 1.0,
+    }
+    params = {k: v.to(dtype) for k, v in params.items()}
+    return {"x": x, "dout": dout, "mask": _pair_mask(b, n, n_masked), "params": params}
+
+
+def triangle_multiplication_inputs(b=1, n=12, dim=64, n_masked=2, dtype=torch.float32, seed=0):
+    """As :func:`triangle_attention_inputs` for ``TriangleMultiplication`` (``dim_hidden = dim``)."""
+    gen = torch.Generator().manual_seed(seed)
+    x = _randn(gen, b, n, n, dim).to(dtype)
+    dout = _randn(gen, b, n, n, dim).to(dtype)
+    params = {
+        "combined.WEIGHT": 1 + 0.1 * _randn(gen, dim), "combined.BIAS": 0.1 * _randn(gen, dim),
+        "combined.linear_weight": _randn(gen, dim, 5 * dim) * dim ** -0.5,
+        "combined.linear_bias": 0.1 * _randn(gen, 5 * dim),
+        "to_out.0.WEIGHT": 1 + 0.1 * _randn(gen, dim), "to_out.0.BIAS": 0.1 * _randn(gen, dim),
+        "to_out.0.linear_weight": _randn(gen, dim, dim) * dim ** -0.5,
+    }
+    params = {k: v.to(dtype) for k, v in params.items()}
+    return {"x": x, "dout": dout, "mask": _pair_mask(b, n, n_masked), "params": params}

@@ -21,6 +21,8 @@ from megafold_amd import workloads  # noqa: E402
 from oracle import evoattention as oe  # noqa: E402
 from oracle import layernorm_linear as ol  # noqa: E402
 from oracle import transition as ot  # noqa: E402
+from oracle import triangle_attention as ota  # noqa: E402
+from oracle import triangle_multiplication as otm  # noqa: E402
 
 f64 = torch.float64
 
@@ -61,7 +63,25 @@ def transition_small():
     np.savez_compressed(os.path.join(HERE, "transition_small.npz"), h=h.numpy(), y=y.numpy())
 
 
+def triangle_blocks_small():
+    """fwd+bwd of the two pair-stack blocks on small ragged shapes, fp32 inputs, both variants each."""
+    out = {}
+    for node in ("starting", "ending"):
+        w = workloads.triangle_attention_inputs(seed=11)
+        o, dx, dp = ota.triangle_attention_forward_backward(w["x"], w["mask"], w["params"], w["dout"], 2, 16, node)
+        out["attn_%s_out" % node], out["attn_%s_dx" % node] = o.numpy(), dx.numpy()
+        out["attn_%s_dWkv" % node] = dp["fn.attn.to_kv.weight"].numpy()
+        out["attn_%s_dWb" % node] = dp["fn.to_attn_bias.0.weight"].numpy()
+    for mix in ("outgoing", "incoming"):
+        w = workloads.triangle_multiplication_inputs(seed=13)
+        o, dx, dp = otm.triangle_multiplication_forward_backward(w["x"], w["mask"], w["params"], w["dout"], mix)
+        out["mult_%s_out" % mix], out["mult_%s_dx" % mix] = o.numpy(), dx.numpy()
+        out["mult_%s_dW1" % mix] = dp["combined.linear_weight"].numpy()
+    np.savez_compressed(os.path.join(HERE, "triangle_blocks_small.npz"), **{k: v.astype(np.float32) for k, v in out.items()})
+
+
 if __name__ == "__main__":
+    triangle_blocks_small()
     attention_c1()
     attention_small_bwd()
     lnlinear_small()

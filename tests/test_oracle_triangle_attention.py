@@ -157,3 +157,15 @@ def test_fused_module_has_the_reference_parameter_names(node_type):
     assert torch.all(sd["fn.attn.to_gates.weight"] == 0) and torch.all(sd["fn.attn.to_gates.bias"] == -2.0)
     with pytest.raises(RuntimeError):
         m(torch.zeros(1, 4, 4, 128))          # no CPU path
+
+
+@pytest.mark.parametrize("node_type", ["starting", "ending"])
+def test_golden_fixture_reproduces(node_type):
+    import os
+    import numpy as np
+    from megafold_amd import workloads
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "triangle_blocks_small.npz"))
+    w = workloads.triangle_attention_inputs(seed=11)
+    out, dx, dp = ota.triangle_attention_forward_backward(w["x"], w["mask"], w["params"], w["dout"], 2, 16, node_type)
+    for name, got in (("out", out), ("dx", dx), ("dWkv", dp["fn.attn.to_kv.weight"]), ("dWb", dp["fn.to_attn_bias.0.weight"])):
+        torch.testing.assert_close(got.float(), torch.from_numpy(g["attn_%s_%s" % (node_type, name)]), rtol=1e-5, atol=1e-6)

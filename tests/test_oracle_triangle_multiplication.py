@@ -131,3 +131,15 @@ def test_fused_module_has_the_reference_parameter_names(mix):
     assert sd["combined.linear_weight"].shape == (128, 640) and sd["to_out.0.linear_weight"].shape == (128, 128)
     with pytest.raises(RuntimeError):
         m(torch.zeros(1, 4, 4, 128))          # no CPU path
+
+
+@pytest.mark.parametrize("mix", ["outgoing", "incoming"])
+def test_golden_fixture_reproduces(mix):
+    import os
+    import numpy as np
+    from megafold_amd import workloads
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "triangle_blocks_small.npz"))
+    w = workloads.triangle_multiplication_inputs(seed=13)
+    out, dx, dp = otm.triangle_multiplication_forward_backward(w["x"], w["mask"], w["params"], w["dout"], mix)
+    for name, got in (("out", out), ("dx", dx), ("dW1", dp["combined.linear_weight"])):
+        torch.testing.assert_close(got.float(), torch.from_numpy(g["mult_%s_%s" % (mix, name)]), rtol=1e-5, atol=1e-6)

@@ -123,3 +123,24 @@ def test_sigmoid_gate_kernels(dtype, M, C, ld):
     torch.testing.assert_close(dO.cpu().double(), do64, **tol)
     torch.testing.assert_close(dY[:, off:].cpu().double(), dg64, **tol)
     assert torch.all(dY[:, :off] == 7.0)        # columns outside the slice are untouched
+
+
+@pytest.mark.parametrize("node_type", ["starting", "ending"])
+def test_block_against_golden_fixture(node_type):
+    """fp32 run against the frozen oracle outputs (tests/golden/triangle_blocks_small.npz)."""
+    import os
+    import numpy as np
+    from megafold_amd import workloads
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "triangle_blocks_small.npz"))
+    w = workloads.triangle_attention_inputs(seed=11)
+    m = PreLayerNormTriangleAttention(dim=64, heads=2, node_type=node_type, dim_head=16)
+    m.load_state_dict(w["params"])
+    m = m.cuda()
+    x = w["x"].cuda().requires_grad_(True)
+    out = m(x, w["mask"].cuda())
+    out.backward(w["dout"].cuda())
+    got = {"out": out, "dx": x.grad, "dWkv": m.fn.attn.to_kv.weight.grad, "dWb": m.fn.to_attn_bias[0].weight.grad}
+    for name, t in got.items():
+        want = torch.from_numpy(g["attn_%s_%s" % (node_type, name)])
+        s = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(t.detach().cpu() / s, want / s, rtol=1e-4, atol=1e-5, msg=lambda m_, n=name: "%s: %s" % (n, m_))

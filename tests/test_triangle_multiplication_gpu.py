@@ -141,3 +141,24 @@ def test_block_under_autocast_with_fp32_master_weights():
     assert all(p.grad is not None and p.grad.dtype == torch.float32 and torch.isfinite(p.grad).all() for p in m.parameters())
     want = otm.triangle_multiplication_forward(x.detach().cpu(), None, {k: v.cpu() for k, v in m.state_dict().items()}, "outgoing")
     torch.testing.assert_close(out.detach().cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("mix", ["outgoing", "incoming"])
+def test_block_against_golden_fixture(mix):
+    """fp32 run against the frozen oracle outputs (tests/golden/triangle_blocks_small.npz)."""
+    import os
+    import numpy as np
+    from megafold_amd import workloads
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "triangle_blocks_small.npz"))
+    w = workloads.triangle_multiplication_inputs(seed=13)
+    m = TriangleMultiplication(dim=64, mix=mix)
+    m.load_state_dict(w["params"])
+    m = m.cuda()
+    x = w["x"].cuda().requires_grad_(True)
+    out = m(x, w["mask"].cuda())
+    out.backward(w["dout"].cuda())
+    got = {"out": out, "dx": x.grad, "dW1": m.combined.linear_weight.grad}
+    for name, t in got.items():
+        want = torch.from_numpy(g["mult_%s_%s" % (mix, name)])
+        s = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(t.detach().cpu() / s, want / s, rtol=1e-4, atol=1e-5, msg=lambda m_, n=name: "%s: %s" % (n, m_))
