@@ -47,48 +47,60 @@ hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t strea
 // =================================================================================================
 // weight preparation:  W' = gamma (.) W in both layouts, column sums of W', folded bias
 // =================================================================================================
-// One work-group owns 16 columns of W and all K rows: reads and writes of the [K, N] layout are
-// coalesced along n, the transposed [N, KP] copy goes through LDS so its rows are written whole.
+// One work-group owns 32 columns of W and all K rows.  A thread moves 8 consecutive columns (16 bytes for
+// the 16-bit types) of every 64th row, so four neighbouring threads read and write 64 contiguous bytes of
+// the [K, N] layout; the transposed [N, KP] copy goes through LDS so that its rows are written whole.
 template <typename T>
 __global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
-  __shared__ float tile[16][257];     // [n][k], K <= 256
-  __shared__ float red_cs[16][17], red_bp[16][17];
-  const int tid = threadIdx.x, nn = tid & 15, kk = tid >> 4;
-  const int n = blockIdx.x * 16 + nn;
+  constexpr int CW = 32;                      // columns per work-group
+  __shared__ float tile[CW][257];             // [n][k], K <= 256
+  __shared__ float red_cs[64][CW + 1], red_bp[64][CW + 1];
+  const int tid = threadIdx.x, c8 = tid & 3, kr = tid >> 2;
+  const int n0 = blockIdx.x * CW + 8 * c8;    // first of this thread's 8 columns (N is a multiple of 8)
   const T* W = reinterpret_cast<const T*>(p.W);
   const T* gamma = reinterpret_cast<const T*>(p.gamma);
   const T* beta = reinterpret_cast<const T*>(p.beta);
   T* Wt = reinterpret_cast<T*>(p.Wt);
   T* Wg = reinterpret_cast<T*>(p.Wg);
-  float cs = 0.0f, bp = 0.0f;
-  for (int k = kk; k < p.KP; k += 16) {
-    float gwf = 0.0f;
-    if (k < p.K && n < p.N) {
-      const float w = to_f(W[(int64_t)k * p.N + n]);
-      const T gw = (T)(to_f(gamma[k]) * w);
-      if (Wg) Wg[(int64_t)k * p.N + n] = gw;
-      gwf = to_f(gw);
-      cs += gwf;
-      if (beta) bp += to_f(beta[k]) * w;
+  float cs[8], bp[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { cs[e] = 0.0f; bp[e] = 0.0f; }
+  for (int k = kr; k < p.KP; k += 64) {
+    float gwf[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) gwf[e] = 0.0f;
+    if (k < p.K && n0 < p.N) {
+      const frag_t<T> w = ld8<T>(W + (int64_t)k * p.N + n0);
+      const float gk = to_f(gamma[k]), bk = beta ? to_f(beta[k]) : 0.0f;
+      frag_t<T> gw;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        gw[e] = (T)(gk * to_f(w[e]));
+        gwf[e] = to_f(gw[e]);
+        cs[e] += gwf[e];
+        bp[e] += bk * to_f(w[e]);
+      }
+      if (Wg) st8<T>(Wg + (int64_t)k * p.N + n0, gw);
     }
-    tile[nn][k] = gwf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tile[8 * c8 + e][k] = gwf[e];
   }
-  red_cs[nn][kk] = cs;
-  red_bp[nn][kk] = bp;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { red_cs[kr][8 * c8 + e] = cs[e]; red_bp[kr][8 * c8 + e] = bp[e]; }
   __syncthreads();
-  if (tid < 16) {
-    const int n2 = blockIdx.x * 16 + tid;
+  if (tid < CW) {
+    const int n2 = blockIdx.x * CW + tid;
     float a = 0.0f, b2 = 0.0f;
-    for (int j = 0; j < 16; ++j) { a += red_cs[tid][j]; b2 += red_bp[tid][j]; }
+    for (int j = 0; j < 64; ++j) { a += red_cs[j][tid]; b2 += red_bp[j][tid]; }   // fixed order
     if (n2 < p.N) {
       if (p.colsum) p.colsum[n2] = a;
       if (p.bprime) p.bprime[n2] = b2 + (p.b ? to_f(reinterpret_cast<const T*>(p.b)[n2]) : 0.0f);
     }
   }
   if (Wt) {
-    for (int i = tid; i < 16 * p.KP; i += 256) {
+    for (int i = tid; i < CW * p.KP; i += 256) {
       const int r = i / p.KP, k = i % p.KP;
-      const int n2 = blockIdx.x * 16 + r;
+      const int n2 = blockIdx.x * CW + r;
       if (n2 < p.N) Wt[(int64_t)n2 * p.KP + k] = (T)tile[r][k];
     }
   }
@@ -96,7 +108,7 @@ __global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
 
 hipError_t launch_ln_prep(const LnParams& p, bool forward, hipStream_t stream) {
   (void)forward;
-  const unsigned blocks = (unsigned)((p.N + 15) / 16);
+  const unsigned blocks = (unsigned)((p.N + 31) / 32);
   switch (p.dtype) {
     case MF_BF16: hipLaunchKernelGGL(ln_prep_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, p); break;
     case MF_F16: hipLaunchKernelGGL(ln_prep_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, p); break;

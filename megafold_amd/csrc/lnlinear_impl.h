@@ -1050,10 +1050,17 @@ __global__ void __launch_bounds__(256) ln_bwd_finalize_kernel(const LnParams p) 
   const float bet = p.beta ? to_f(reinterpret_cast<const T*>(p.beta)[k]) : 0.0f;
   float dg = 0.0f, dbt = 0.0f;
   for (int n = tid; n < p.N; n += 256) {
-    float G = 0.0f;
     const int64_t kn = (int64_t)p.K * p.N;
     const int nr = p.R < LN_RED_GROUPS ? p.R : LN_RED_GROUPS;
-    for (int r = 0; r < nr; ++r) G += p.Gpart[(int64_t)r * kn + (int64_t)k * p.N + n];   // fixed order
+    // all loads first (independent), then the sum in its fixed order: a load-add chain would pay the
+    // memory latency once per range
+    float gv[LN_RED_GROUPS];
+#pragma unroll
+    for (int r = 0; r < LN_RED_GROUPS; ++r)
+      gv[r] = r < nr ? p.Gpart[(int64_t)r * kn + (int64_t)k * p.N + n] : 0.0f;
+    float G = 0.0f;
+#pragma unroll
+    for (int r = 0; r < LN_RED_GROUPS; ++r) G += gv[r];
     const float s = p.spart[n];
     const float wv = to_f(W[(int64_t)k * p.N + n]);
     p.dW[(int64_t)k * p.N + n] = gam * G + bet * s;
