@@ -55,21 +55,27 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write(out + "\n")
 
 
+# sources whose MFMAs are inline assembly: the compiler does not see their hazards
+ASM_MFMA_SOURCES = ("evoattn_bwd_pw", "evoattn_bwd_dbias_ring")
+
+
 def _check_generated_code(hipcc: str, extra: list[str]) -> None:
-    """evoattn_bwd_pw.hip issues its MFMAs as inline assembly, which hides them from the compiler's hazard
-    handling; csrc/check_pw_hazards.py verifies the required distances on the generated assembly text."""
-    src = CSRC / "evoattn_bwd_pw.hip"
-    asm = OBJ / "evoattn_bwd_pw.s"
-    _run([hipcc, *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src.stem, []), *extra, "-S", "--cuda-device-only", str(src),
-          "-o", str(asm)])
+    """evoattn_bwd_pw.hip and evoattn_bwd_dbias_ring.hip issue their MFMAs as inline assembly, which hides them
+    from the compiler's hazard handling; csrc/check_pw_hazards.py verifies the required distances on the
+    generated assembly text."""
     sys.path.insert(0, str(CSRC))
     try:
         import check_pw_hazards
-        errs = check_pw_hazards.check(str(asm))
     finally:
         sys.path.pop(0)
-    if errs:
-        raise RuntimeError("hazards in the generated code of %s:\n%s" % (src.name, "\n".join(errs[:20])))
+    for stem in ASM_MFMA_SOURCES:
+        src = CSRC / (stem + ".hip")
+        asm = OBJ / (stem + ".s")
+        _run([hipcc, *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src.stem, []), *extra, "-S", "--cuda-device-only", str(src),
+              "-o", str(asm)])
+        errs = check_pw_hazards.check(str(asm))
+        if errs:
+            raise RuntimeError("hazards in the generated code of %s:\n%s" % (src.name, "\n".join(errs[:20])))
 
 
 def build(verbose: bool = False, jobs: int | None = None) -> Path:

@@ -1,6 +1,6 @@
-"""Checks the generated code of evoattn_bwd_pw.hip for hazards the compiler cannot see.
+"""Checks the generated code of evoattn_bwd_pw.hip and evoattn_bwd_dbias_ring.hip for hazards the compiler cannot see.
 
-The kernel issues its MFMAs as inline assembly, so the compiler neither inserts the idle cycles gfx950
+These kernels issue their MFMAs as inline assembly, so the compiler neither inserts the idle cycles gfx950
 requires around them nor keeps their operands alive long enough.  This script reads the assembly text the
 compiler produced (``hipcc -S``) and verifies, for every MFMA inside an ``#ASMSTART`` / ``#ASMEND`` pair:
 
@@ -91,42 +91,51 @@ def check(path: str) -> list[str]:
 
 
 N_CHECKED = [0]
+# kernels (substrings of the mangled names) whose inline-assembly MFMAs are checked
+CHECKED_KERNELS = ("dqkv_pw", "dbias_ring")
 
 
-def forward(insts, i, limit):
-    """Instructions after position i with the smallest number of issue slots that can separate them from
-    it: a conditional branch to a later label may be taken, so the instructions it skips are visited (they
-    may execute) but do not add to the count.  Stops at `limit` slots, at backward or unconditional branches."""
+def paths(insts, i, limit):
+    """Every instruction sequence that can follow position i, as lists of (instruction, issue slots that separate
+    it from position i): at a conditional branch to a later label both continuations are followed.  A sequence ends
+    after `limit` slots, at a backward or unconditional branch, or at the end of the program."""
     labels = {t: k for k, (m, _, _, _, t, _) in enumerate(insts) if m == "label"}
-    fwd, j, free_until = 0, i + 1, -1
-    while j < len(insts) and fwd < limit:
-        m2, w2, r2, a2, t2, n2 = insts[j]
-        if m2 == "label":
-            j += 1
-            continue
-        if m2 in ("s_branch", "s_endpgm", "s_setpc_b64"):
-            return
-        if m2.startswith("s_cbranch"):
-            target = labels.get(t2.split()[-1])
-            if target is None or target <= j:
-                return
-            free_until = max(free_until, target)
-            j += 1
-            continue
-        yield insts[j], fwd
-        if j > free_until:
+    out = []
+    todo = [(i + 1, 0, [])]
+    while todo:
+        j, fwd, seq = todo.pop()
+        seq = list(seq)
+        while j < len(insts) and fwd < limit:
+            m2, w2, r2, a2, t2, n2 = insts[j]
+            if m2 == "label":
+                j += 1
+                continue
+            if m2 in ("s_branch", "s_endpgm", "s_setpc_b64"):
+                break
+            if m2.startswith("s_cbranch"):
+                target = labels.get(t2.split()[-1])
+                if target is None or target <= j:
+                    break
+                if len(todo) < 64:
+                    todo.append((target, fwd, list(seq)))
+                j += 1
+                continue
+            seq.append((insts[j], fwd))
             fwd += slots(m2, t2)
-        j += 1
+            j += 1
+        out.append(seq)
+    return out
 
 
 def check_kernel(kernel: str, insts) -> list[str]:
     errors = []
-    if "dqkv_pw" not in kernel:
+    if not any(name in kernel for name in CHECKED_KERNELS):
         return errors
     for i, (mnem, wr, rd, in_asm, text, no) in enumerate(insts):
         if not (in_asm and mnem.startswith("v_mfma")):
             continue
         N_CHECKED[0] += 1
+        found = set()      # two paths may report the same instruction
         ops = [o.strip() for o in text.split(None, 1)[1].split(",")]
         dst, srcc = regs(ops[0]), regs(ops[3]) if len(ops) > 3 else set()
         # 1. vector-ALU writes of operands in the two preceding slots
@@ -141,32 +150,36 @@ def check_kernel(kernel: str, insts) -> list[str]:
             j -= 1
         # 2. C operand rewritten while the product runs
         if srcc and srcc != dst:
-            for (m2, w2, r2, a2, t2, n2), fwd in forward(insts, i, 13):
-                if w2 & srcc:
-                    errors.append("%s: line %d `%s` rewrites the C operand of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
+            for seq in paths(insts, i, 13):
+                for (m2, w2, r2, a2, t2, n2), fwd in seq:
+                    if w2 & srcc:
+                        found.add("%s: line %d `%s` rewrites the C operand of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
         # 3. vector-register result read too early (12 slots, two of them MFMAs or idle instructions; 24 slots
         #    of any kind are as good).  A register that another instruction has rewritten no longer holds the result.
         if any(k == "v" for k, _ in dst):
-            busy, live = 0, set(dst)
-            for (m2, w2, r2, a2, t2, n2), fwd in forward(insts, i, 1 << 30):
-                if (fwd >= 12 and busy >= 2) or fwd >= 24 or not live:
-                    break
-                if (r2 & live) and not m2.startswith("v_mfma"):
-                    errors.append("%s: line %d `%s` reads the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
-                    break
-                if not m2.startswith("v_mfma"):
-                    if (w2 & live) and fwd < 12:
-                        errors.append("%s: line %d `%s` overwrites the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
+            for seq in paths(insts, i, 26):
+                busy, live = 0, set(dst)
+                for (m2, w2, r2, a2, t2, n2), fwd in seq:
+                    if (fwd >= 12 and busy >= 2) or fwd >= 24 or not live:
                         break
-                    live -= w2
-                if m2.startswith("v_mfma") or m2 == "s_nop":
-                    busy += 1
+                    if (r2 & live) and not m2.startswith("v_mfma"):
+                        found.add("%s: line %d `%s` reads the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
+                        break
+                    if not m2.startswith("v_mfma"):
+                        if (w2 & live) and fwd < 12:
+                            found.add("%s: line %d `%s` overwrites the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
+                            break
+                        live -= w2
+                    if m2.startswith("v_mfma") or m2 == "s_nop":
+                        busy += 1
         # 4. accumulation-register result read by something other than an MFMA
         if any(k == "a" for k, _ in dst):
-            for (m2, w2, r2, a2, t2, n2), fwd in forward(insts, i, 18):
-                if (r2 & dst) and not m2.startswith("v_mfma"):
-                    errors.append("%s: line %d `%s` reads the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
-                    break
+            for seq in paths(insts, i, 18):
+                for (m2, w2, r2, a2, t2, n2), fwd in seq:
+                    if (r2 & dst) and not m2.startswith("v_mfma"):
+                        found.add("%s: line %d `%s` reads the result of the MFMA at line %d after %d slots" % (kernel, n2, t2, no, fwd))
+                        break
+        errors += sorted(found)
     return errors
 
 

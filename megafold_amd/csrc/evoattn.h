@@ -55,6 +55,11 @@ struct EvoParams {
 hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dbias(const EvoParams& p, hipStream_t stream);
+// Bias-gradient kernel that streams its rows through an LDS ring with direct loads (16-bit, D = 32, paired heads;
+// evoattn_bwd_dbias_ring.hip): whether it handles the problem, and its launcher (same grid and chunking as
+// the paired-head form of evo_bwd_dbias_kernel; the caller sums the partial buffers).
+bool evo_bwd_dbias_ring_supported(const EvoParams& p);
+hipError_t launch_evo_bwd_dbias_ring(const EvoParams& p, hipStream_t stream);
 // Persistent form of the dQ/dK/dV kernel (16-bit element types, D <= 32; evoattn_bwd_pw.hip): whether it
 // handles the problem, and its launcher (num_cu = compute units of the device).
 // Compute units of the current device (256 when no device can be queried).

@@ -1168,6 +1168,18 @@ int evo_dbias_chunks(int B, int N, int S, int H, int D, int dtype) {
   return best;
 }
 
+// Fixed-order sum of the chunks' partial buffers (nothing to do with one chunk: the kernel wrote dbias itself).
+static hipError_t launch_dbias_reduce(const EvoParams& p, hipStream_t stream) {
+  if (p.n_chunks <= 1) return hipSuccess;
+  const int64_t n = (int64_t)p.B * p.H * p.S * p.S;
+  const int vec = (n & 3) == 0;     // partial buffers and dbias are 16-byte aligned
+  int64_t rb = ((vec ? n >> 2 : n) + 255) / 256;
+  if (rb > 2048) rb = 2048;
+  hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)rb), dim3(256), 0, stream, p.dbias_part, p.dbias, n,
+                     p.n_chunks, vec);
+  return hipGetLastError();
+}
+
 template <typename T, int DP, int TR, int HP> static hipError_t launch_dbias_t(const EvoParams& p, hipStream_t stream) {
   using L = BwdLayout<T, DP>;
   const int NT = (p.S + 31) / 32;
@@ -1186,16 +1198,7 @@ template <typename T, int DP, int TR, int HP> static hipError_t launch_dbias_t(c
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256 * HP), smem, stream, p, IB, JB);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  if (p.n_chunks > 1) {
-    const int64_t n = (int64_t)p.B * p.H * p.S * p.S;
-    const int vec = (n & 3) == 0;     // partial buffers and dbias are 16-byte aligned
-    int64_t rb = ((vec ? n >> 2 : n) + 255) / 256;
-    if (rb > 2048) rb = 2048;
-    hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)rb), dim3(256), 0, stream, p.dbias_part, p.dbias, n,
-                       p.n_chunks, vec);
-    e = hipGetLastError();
-  }
-  return e;
+  return launch_dbias_reduce(p, stream);
 }
 
 template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipStream_t stream) {
@@ -1203,8 +1206,15 @@ template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipSt
   if constexpr (!wide) {
     // whole-line staging of a head pair needs the two heads side by side in memory (D = 32 exactly)
     if (dbias_pairs_heads(p.dtype, p.D, p.H) && p.D == 32 && p.q.sh == 32 && p.k.sh == 32 && p.v.sh == 32 &&
-        p.dO.sh == 32)
+        p.dO.sh == 32) {
+#ifndef MF_NO_DBIAS_RING
+      if (evo_bwd_dbias_ring_supported(p)) {
+        const hipError_t e = launch_evo_bwd_dbias_ring(p, stream);
+        return e != hipSuccess ? e : launch_dbias_reduce(p, stream);
+      }
+#endif
       return launch_dbias_t<T, 32, 2, 2>(p, stream);
+    }
   }
   if (p.D <= 32) return launch_dbias_t<T, 32, wide ? 1 : 2, 1>(p, stream);
   if (p.D <= 64) return launch_dbias_t<T, 64, 1, 1>(p, stream);

@@ -58,3 +58,19 @@ def test_accumulation_register_result_read_by_other_units(tmp_path):
     assert any("reads the result" in e for e in run(tmp_path, bad))
     good = asm(MFMA_A) + "s_nop 15\ns_nop 3\nds_write_b128 v90, a[16:19]\n"
     assert run(tmp_path, good) == []
+
+
+def test_conditional_branch_both_continuations_are_followed(tmp_path):
+    """A reader inside a conditionally skipped region is separated from the product by the region's own
+    instructions; a reader behind the branch target is not (the branch may be taken)."""
+    filler = "v_add_f32_e32 v80, v81, v82\n" * 10 + "s_nop 1\ns_nop 1\n"
+    inside = asm(MFMA_V) + "s_cbranch_scc1 .LBB0_9\n" + filler + "v_mul_f32_e32 v60, v61, v3\n.LBB0_9:\ns_endpgm\n"
+    assert run(tmp_path, inside) == []
+    behind = asm(MFMA_V) + "s_cbranch_scc1 .LBB0_9\n" + filler + ".LBB0_9:\nv_mul_f32_e32 v60, v61, v3\ns_endpgm\n"
+    assert any("reads the result" in e for e in run(tmp_path, behind))
+
+
+def test_bias_gradient_ring_kernel_is_checked(tmp_path):
+    f = tmp_path / "k.s"
+    f.write_text("_ZN2mf25evo_bwd_dbias_ring_kernelIDF16bLi4EEEvNS_9EvoParamsEii:\n" + asm(MFMA_V) + "v_mul_f32_e32 v60, v61, v3\n")
+    assert any("reads the result" in e for e in chk.check(str(f)))
