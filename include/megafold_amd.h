@@ -72,7 +72,9 @@ const char* mf_last_error(void);
  * MF_EVO_BWD_DQKV needs that copy, writes dq, dk, dv and leaves rowsum(dO * o) in the workspace;
  * MF_EVO_BWD_DBIAS needs both and writes dbias.  A call with a subset of the phases must therefore
  * follow calls for the earlier ones on the same stream with the same workspace.  phases = 0 runs
- * all of them (DBIAS only when dbias != NULL). */
+ * all of them (DBIAS only when dbias != NULL).
+ * The workspace size depends on the shape, on whether dbias is requested and on the number of compute units of
+ * the CURRENT device: query it with the arguments of the call and with the device of the call current. */
 #define MF_EVO_BWD_DQKV 1
 #define MF_EVO_BWD_DBIAS 2
 #define MF_EVO_BWD_PREP 4

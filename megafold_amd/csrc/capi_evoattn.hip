@@ -35,7 +35,8 @@ Plan make_plan(const mf_evoattn_args* a, bool backward) {
     if (a->dbias) {
       pl.n_chunks = evo_dbias_chunks(a->B, a->N, a->S, a->H, a->D, a->dtype);
       pl.rows_per_chunk = (a->N + pl.n_chunks - 1) / pl.n_chunks;
-      if (pl.n_chunks > 1) part_bytes = (uint64_t)pl.n_chunks * a->B * a->H * a->S * a->S * 4;
+      // the first chunk writes into dbias itself
+      if (pl.n_chunks > 1) part_bytes = (uint64_t)(pl.n_chunks - 1) * a->B * a->H * a->S * a->S * 4;
     }
     // the multi-pass dQ array of the dQ/dK/dV kernel is dead before the bias-gradient kernel starts: one region
     pl.dq_scratch_bytes = evo_bwd_dqkv_pw_scratch_bytes(a->dtype, a->S, a->D, evo_num_cu());

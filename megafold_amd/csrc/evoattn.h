@@ -40,7 +40,7 @@ struct EvoParams {
   EvoTensor dO, dq, dk, dv;
   float* delta;    // [B, N, H, S] fp32 rowsum(dO * O)
   float* dbias;    // [B, H, S, S] fp32 or nullptr
-  float* dbias_part;  // [n_chunks, B, H, S, S] fp32 partial sums (nullptr when n_chunks == 1)
+  float* dbias_part;  // [n_chunks - 1, B, H, S, S] fp32 partial sums of the chunks 1.. (chunk 0 writes dbias; nullptr when n_chunks == 1)
   float* dq_scratch;  // fp32 dQ of the sequences the persistent dQ/dK/dV kernel walks in several passes: one
                       // [ceil(S/32) * 32, 32] array per work-group (evo_bwd_dqkv_pw_scratch_bytes), else nullptr
 #ifdef MF_TIMELINE

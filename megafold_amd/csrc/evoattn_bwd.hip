@@ -1068,7 +1068,8 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   }
 
   // ---- store the patch: lane (x = query, g) owns 16 contiguous keys per tile ---------------------
-  float* dst = (p.n_chunks > 1 ? p.dbias_part + (int64_t)chunk * p.B * p.H * S * S : p.dbias) +
+  // chunk 0 writes into dbias itself, the others into the partial buffers that the reduction adds to it
+  float* dst = (chunk > 0 ? p.dbias_part + (int64_t)(chunk - 1) * p.B * p.H * S * S : p.dbias) +
                ((int64_t)b * p.H + h) * S * S;
   if (qi < S) {
     const bool vec = (S & 3) == 0;     // rows of the gradient are 16-byte aligned
@@ -1090,17 +1091,19 @@ evo_bwd_dbias_kernel(const EvoParams p, const int IB, const int JB) {
   }
 }
 
-// out = sum over chunks of part[c], four elements per thread when `vec` (n a multiple of 4).
-__global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, float* out, int64_t n, int chunks, int vec) {
+// out += sum over the partial buffers part[0 .. parts), in that order (out holds the first chunk's sum); four
+// elements per thread when `vec` (n a multiple of 4).
+__global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, float* out, int64_t n, int parts, int vec) {
   if (vec) {
     const int64_t n4 = n >> 2;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
-      // chunks <= 8: all loads are issued together, the sum keeps its fixed order
+      // parts <= 7: all loads are issued together, the sum keeps its fixed order
       f32x4 v[8];
+      v[0] = *reinterpret_cast<const f32x4*>(out + 4 * i);
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
+      for (int c = 1; c < 8; ++c) {
         const f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
-        v[c] = c < chunks ? *reinterpret_cast<const f32x4*>(part + (int64_t)c * n + 4 * i) : z;
+        v[c] = c <= parts ? *reinterpret_cast<const f32x4*>(part + (int64_t)(c - 1) * n + 4 * i) : z;
       }
       f32x4 s = v[0];
 #pragma unroll
@@ -1110,8 +1113,9 @@ __global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, fl
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
       float v[8];
+      v[0] = out[i];
 #pragma unroll
-      for (int c = 0; c < 8; ++c) v[c] = c < chunks ? part[(int64_t)c * n + i] : 0.0f;
+      for (int c = 1; c < 8; ++c) v[c] = c <= parts ? part[(int64_t)(c - 1) * n + i] : 0.0f;
       float s = v[0];
 #pragma unroll
       for (int c = 1; c < 8; ++c) s += v[c];
@@ -1176,7 +1180,7 @@ static hipError_t launch_dbias_reduce(const EvoParams& p, hipStream_t stream) {
   int64_t rb = ((vec ? n >> 2 : n) + 255) / 256;
   if (rb > 2048) rb = 2048;
   hipLaunchKernelGGL(dbias_reduce_kernel, dim3((unsigned)rb), dim3(256), 0, stream, p.dbias_part, p.dbias, n,
-                     p.n_chunks, vec);
+                     p.n_chunks - 1, vec);
   return hipGetLastError();
 }
 

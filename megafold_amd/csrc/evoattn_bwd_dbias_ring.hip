@@ -37,7 +37,7 @@ namespace {
 // LDS: three row slots, the key side of all slots first (so that every key-side read of a lane is one address
 // register plus an immediate), then the query side.  Byte offsets:
 constexpr int KS_BYTES = 16640;  // key side of one slot
-constexpr int KS_K = 0;          //   [64 key rows][2 heads x 64 bytes], chunk c of row m at position c ^ (m & 7)
+constexpr int KS_K = 0;          //   [64 key rows][2 heads x 64 bytes], chunk c of row m at position c ^ ((m >> 1) & 7)
 constexpr int KS_V = 8192;
 constexpr int KS_MK = 16384;     //   [64 key rows] packed (hi, lo) of mask / scale
 constexpr int QS_BASE = 3 * KS_BYTES;
@@ -48,7 +48,11 @@ constexpr int QS_Q = 2048;       //   [128 query rows][2 heads x 64 bytes], same
 constexpr int QS_DO = 18432;
 constexpr int RING_BYTES = QS_BASE + 3 * QS_BYTES;
 constexpr int RING = 3;
+#ifdef MF_RING_KO_DO      // timing experiment, wrong results: dO is not loaded
+constexpr int ROW_OPS = 5;
+#else
 constexpr int ROW_OPS = 7;       // direct-to-LDS loads per wavefront and row
+#endif
 
 #define MF_SB() __builtin_amdgcn_sched_barrier(0)
 
@@ -157,7 +161,7 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
 
   // ---- per-lane byte offsets of the direct loads (relative to the row's base address) ------------------
   const int es = (int)sizeof(T);
-  const int m = t512 >> 3, pos = t512 & 7, cg = pos ^ (m & 7);   // LDS row, position, global chunk that lands there
+  const int m = t512 >> 3, pos = t512 & 7, cg = pos ^ ((m >> 1) & 7);   // LDS row, position, global chunk that lands there
   unsigned koff, voff, qoff[2], dooff[2];
   {
     int key = jt0 * 32 + (m & 32) + unperm32(m & 31);
@@ -203,21 +207,34 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
   const unsigned wslot = (unsigned)wv * 1024;
   const unsigned ldst = QS_BASE + (wv < 4 ? QS_LSE : QS_DL) + (unsigned)(wv & 3) * 256;
 
-  // request one row into ring slot `slot`; past the chunk's last row the last row is requested again
-  auto issue_row = [&](int slot) {
+  // Request of one row into ring slot `slot`, in seven parts (one instruction each) so that the requests can be
+  // spread over a row step: a wavefront that issues them in one burst sits in the memory pipeline's queue for
+  // hundreds of cycles.  Past the chunk's last row the last row is requested again.
+  auto issue_part = [&](int slot, int part) {
     const unsigned ks = lds0 + (unsigned)slot * KS_BYTES + wslot;
     const unsigned qs = lds0 + QS_BASE + (unsigned)slot * QS_BYTES + wslot;
-    dma16(koff, kb, ks + KS_K);
-    dma16(voff, vb, ks + KS_V);
-    dma16(qoff[0], qb, qs + QS_Q);
-    dma16(qoff[1], qb, qs + QS_Q + 8192);
-    dma16(dooff[0], dob, qs + QS_DO);
-    dma16(dooff[1], dob, qs + QS_DO + 8192);
-    dma4(ldoff, ldb, lds0 + (unsigned)slot * QS_BYTES + ldst);
-    if (rows_left > 0) {
-      kb += k_step; vb += v_step; qb += q_step; dob += do_step; ldb += ld_step;
+    switch (part) {
+      case 0: dma16(koff, kb, ks + KS_K); break;
+      case 1: dma16(voff, vb, ks + KS_V); break;
+      case 2: dma16(qoff[0], qb, qs + QS_Q); break;
+      case 3: dma16(qoff[1], qb, qs + QS_Q + 8192); break;
+#ifndef MF_RING_KO_DO
+      case 4: dma16(dooff[0], dob, qs + QS_DO); break;
+      case 5: dma16(dooff[1], dob, qs + QS_DO + 8192); break;
+#endif
+      case 6:
+        dma4(ldoff, ldb, lds0 + (unsigned)slot * QS_BYTES + ldst);
+        if (rows_left > 0) {
+          kb += k_step; vb += v_step; qb += q_step; dob += do_step; ldb += ld_step;
+        }
+        --rows_left;
+        break;
+      default: break;
     }
-    --rows_left;
+  };
+  auto issue_row = [&](int slot) {
+#pragma unroll
+    for (int part = 0; part < 7; ++part) issue_part(slot, part);
   };
   // the 64 mask elements of a row, raw, one per lane (every wavefront requests them so that all wavefronts
   // count the same number of outstanding loads; the first one converts and publishes them)
@@ -250,8 +267,8 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     const int c = hs * 4 + 2 * g + s;            // 16-byte chunk of the pair line: head hs, d = 16 g + 8 s
-    qa[s] = QS_BASE + QS_Q + qrow * 128 + ((c ^ (qrow & 7)) << 4);
-    ka[s] = KS_K + x * 128 + ((c ^ (x & 7)) << 4);
+    qa[s] = QS_BASE + QS_Q + qrow * 128 + ((c ^ ((qrow >> 1) & 7)) << 4);
+    ka[s] = KS_K + x * 128 + ((c ^ ((x >> 1) & 7)) << 4);
   }
   const int la = QS_BASE + QS_LSE + (hs * 128 + qrow) * 4;
 
@@ -259,7 +276,8 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
   const frag ones_aug = make_aug<T>(ones_g, 0u);
 
   // query-side state of the row being worked on
-  frag qc[2], doc[2], dB;
+  frag qc[2], doc[2];
+  u32x4 dB4 = {0u, 0u, 0u, 0u}, mk4 = {0u, 0u, 0u, 0u};   // carrier fragments: only the first word ever changes
   float l2p;
   auto read_query_side = [&](int slot) {
     const unsigned char* sb = smem + slot * QS_BYTES;
@@ -271,7 +289,7 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
     const float lraw = *reinterpret_cast<const float*>(sb + la);
     const float draw = *reinterpret_cast<const float*>(sb + la + (QS_DL - QS_LSE));
     l2p = (qi < S && lraw != -__builtin_inff()) ? lraw * MF_LOG2E : __builtin_inff();
-    dB = make_aug<T>(g == 0 ? pack_split<T>(-draw) : 0u, 0u);
+    dB4[0] = g == 0 ? pack_split<T>(-draw) : 0u;
   };
   // One tile step: the matrix pipe computes the scores / scale (seeded with the bias, mask through the carrier) and
   // dP - delta of key tile `tn` of the row in `slot` into (zn, dpn) while the vector ALU turns the finished tile
@@ -279,13 +297,14 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
   // independent vector-ALU instructions, one run behind each product; the empty statements keep every run where
   // it is written.  COMPUTE = false: products only (the very first tile).
   using MM = RingMma<T>;
-  auto tile_step = [&](int slot, int tn, f32x16& zn, f32x16& dpn, auto compute_c, int tc, f32x16& zc, f32x16& dpc, float l2) {
+  auto tile_step = [&](int slot, int tn, f32x16& zn, f32x16& dpn, auto compute_c, int tc, f32x16& zc, f32x16& dpc, float l2, auto&& hook) {
     constexpr bool COMPUTE = decltype(compute_c)::value;
     const unsigned char* sb = smem + slot * KS_BYTES + tn * 4096;
     const unsigned mw = *reinterpret_cast<const unsigned*>(smem + slot * KS_BYTES + KS_MK + (32 * tn + x) * 4);
     const frag k0 = lds_frag<T>(sb + ka[0]), k1 = lds_frag<T>(sb + ka[1]);
     const frag v0 = lds_frag<T>(sb + ka[0] + (KS_V - KS_K)), v1 = lds_frag<T>(sb + ka[1] + (KS_V - KS_K));
-    const frag mfrag = make_aug<T>(g == 0 ? mw : 0u, 0u);
+    mk4[0] = g == 0 ? mw : 0u;
+    const frag mfrag = __builtin_bit_cast(frag, mk4), dB = __builtin_bit_cast(frag, dB4);
     auto st_arg = [&](const int o) {
       if constexpr (COMPUTE) {
 #pragma unroll
@@ -307,50 +326,103 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
         asm volatile("" : "+v"(acc[tc]));
       }
     };
+#ifdef MF_RING_KO_MFMA   // timing experiment, wrong results
+    asm volatile("" : "=v"(zn), "=v"(dpn) : "v"(mfrag), "v"(dB), "v"(k0), "v"(k1), "v"(v0), "v"(v1));
+    st_arg(0); hook(0); st_exp(0); hook(1); st_acc(0); hook(2); st_arg(1); hook(3); st_exp(1); hook(4); st_acc(1); hook(5);
+#else
     MM::set(zn, mfrag, ones_aug, bz[tn]);
     st_arg(0);
+    hook(0);
     MM::zero(dpn, ones_aug, dB);
     st_exp(0);
+    hook(1);
     MM::acc(zn, k0, qc[0]);
     st_acc(0);
+    hook(2);
     MM::acc(dpn, v0, doc[0]);
     st_arg(1);
+    hook(3);
     MM::acc(zn, k1, qc[1]);
     st_exp(1);
+    hook(4);
     MM::acc(dpn, v1, doc[1]);
     st_acc(1);
+    hook(5);
+#endif
   };
+#ifdef MF_RING_KO_VALU    // timing experiment, wrong results
+  using yes = std::integral_constant<bool, false>;
+#else
   using yes = std::integral_constant<bool, true>;
+#endif
   using no = std::integral_constant<bool, false>;
 
   // ---- prologue: rows 0, 1, 2 requested, mask of row 0 published, products of (row 0, tile 0) --------------
   f32x16 zA, dpA, zB, dpB;
+  auto no_hook = [](int) {};
   issue_mask();
   issue_row(0);
   issue_row(1);
   wait_vm<2 * ROW_OPS>();
   publish_mask(0);
   issue_mask();
-  issue_row(2);
-  barrier_keep_vm<2 * ROW_OPS + 1>();
+  issue_part(2, 0); issue_part(2, 1); issue_part(2, 2);      // the rest of row 2 follows in the first row step
+  barrier_keep_vm<ROW_OPS + 1 + 3>();
   read_query_side(0);
-  tile_step(0, 0, zA, dpA, no(), 0, zB, dpB, 0.0f);
+  tile_step(0, 0, zA, dpA, no(), 0, zB, dpB, 0.0f, no_hook);
   asm volatile("s_nop 15\n s_nop 15" : "+v"(zA), "+v"(dpA));   // no vector-ALU run sits between these products and their first use
 
+#ifdef MF_TIMELINE
+  // development aid: shader-clock stamps of rows 20..35 of the chosen work-group, logged in LDS behind the ring
+  unsigned* tlog = reinterpret_cast<unsigned*>(smem + RING_BYTES);
+  int tl_row = 0;
+#define MF_RTL(k)                                                                                      \
+  do {                                                                                                 \
+    if (p.tl && (int)blockIdx.x == p.tl_block && l == 0 && tl_row >= 20 && tl_row < 36)                \
+      tlog[((tl_row - 20) * 8 + wv) * 8 + (k)] = (unsigned)__builtin_readcyclecounter();               \
+  } while (0)
+#else
+#define MF_RTL(k) do { } while (0)
+#endif
   // One row step.  SL = ring slot of row n; the barrier in the middle publishes row n + 1 (slot NS) and frees SL.
   auto row_step = [&](auto slot_c) {
-    constexpr int SL = decltype(slot_c)::value, NS = (SL + 1) % RING;
+    constexpr int SL = decltype(slot_c)::value, NS = (SL + 1) % RING, PS = (SL + 2) % RING;
     float l2 = l2p;
     pin(l2);
-    tile_step(SL, 1, zB, dpB, yes(), 0, zA, dpA, l2);
+    MF_RTL(0);
+    // parts 3..6 of row n + 2 (its slot is the one before SL), one behind every other product
+    tile_step(SL, 1, zB, dpB, yes(), 0, zA, dpA, l2, [&](int stage) {
+#ifndef MF_RING_KO_DMA
+      if (stage == 0) issue_part(PS, 3);
+      if (stage == 1) issue_part(PS, 4);
+      if (stage == 3) issue_part(PS, 5);
+      if (stage == 5) issue_part(PS, 6);
+#endif
+    });
+    MF_RTL(1);
     wait_vm<ROW_OPS>();                          // row n + 1 and its mask have arrived, row n + 2 still travels
+    MF_RTL(2);
     publish_mask(NS);
     barrier_keep_vm<ROW_OPS>();
+    MF_RTL(3);
+#ifndef MF_RING_KO_DMA     // timing experiment, wrong results
     issue_mask();                                // row n + 2
-    issue_row(SL);                               // row n + 3
+#endif
     pin(l2);                                     // the second tile's vector-ALU work stays behind the barrier
+    MF_RTL(4);
     read_query_side(NS);
-    tile_step(NS, 0, zA, dpA, yes(), 1, zB, dpB, l2);
+    // parts 0..2 of row n + 3 go into the slot the barrier has just freed
+    tile_step(NS, 0, zA, dpA, yes(), 1, zB, dpB, l2, [&](int stage) {
+#ifndef MF_RING_KO_DMA
+      if (stage == 0) issue_part(SL, 0);
+      if (stage == 2) issue_part(SL, 1);
+      if (stage == 4) issue_part(SL, 2);
+#endif
+    });
+    MF_RTL(5);
+#ifdef MF_TIMELINE
+    ++tl_row;
+#endif
   };
   {
     int r = 0;
@@ -368,10 +440,16 @@ __global__ void __launch_bounds__(512, 1) evo_bwd_dbias_ring_kernel(const EvoPar
   // compiler knows: keep all of them allocated until the matrix pipe has drained, or a register an MFMA in flight
   // reads or writes is handed to the store code below.
   asm volatile("s_nop 15\n s_nop 15" : "+v"(zA), "+v"(dpA), "+v"(bz[0]), "+v"(bz[1]));
+#ifdef MF_TIMELINE
+  __syncthreads();
+  if (p.tl && (int)blockIdx.x == p.tl_block)
+    for (int i = t512; i < 16 * 8 * 8; i += 512) p.tl[i] = tlog[i];
+#endif
   wait_vm<0>();                                  // nothing of this work-group may still travel towards its LDS
 
   // ---- store the patch: lane (x = query, g) owns 16 contiguous keys per tile ---------------------
-  float* dst = (p.n_chunks > 1 ? p.dbias_part + (int64_t)chunk * p.B * p.H * S * S : p.dbias) +
+  // chunk 0 writes into dbias itself, the others into the partial buffers that the reduction adds to it
+  float* dst = (chunk > 0 ? p.dbias_part + (int64_t)(chunk - 1) * p.B * p.H * S * S : p.dbias) +
                ((int64_t)b * p.H + h) * S * S;
   if (qi < S) {
     const bool vec = (S & 3) == 0;     // rows of the gradient are 16-byte aligned
@@ -409,7 +487,11 @@ bool evo_bwd_dbias_ring_supported(const EvoParams& p) {
 template <typename T, int MES> static hipError_t launch_ring_t(const EvoParams& p, hipStream_t stream) {
   const int NT = (p.S + 31) / 32;
   const int IB = (p.S + 127) / 128, JB = (NT + 1) / 2;
+#ifdef MF_TIMELINE
+  const size_t smem = (size_t)RING_BYTES + 4096;
+#else
   const size_t smem = (size_t)RING_BYTES;
+#endif
   const long long blocks = ((long long)p.B * (p.H / 2) * p.n_chunks * IB * JB + 7) / 8 * 8;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
   auto kern = evo_bwd_dbias_ring_kernel<T, MES>;
@@ -436,5 +518,6 @@ hipError_t launch_evo_bwd_dbias_ring(const EvoParams& p, hipStream_t stream) {
 }
 
 #undef MF_SB
+#undef MF_RTL
 
 }  // namespace mf
