@@ -51,7 +51,12 @@ class AttentionPairBias(nn.Module):
         self.to_attn_bias = nn.Sequential(ln_linear, nn.Identity())   # the reference's Rearrange holds no state
 
     def forward(self, single_repr: torch.Tensor, *, pairwise_repr: torch.Tensor,
-                attn_bias: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None, **_unused) -> torch.Tensor:
+                attn_bias: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None, **kwargs) -> torch.Tensor:
+        # keywords the reference forwards to Attention (context, windowed_mask, memory_kv, value_residual, ...)
+        # select paths that are not built here: refuse them instead of computing self-attention silently
+        extra = [k for k, v in kwargs.items() if v is not None and k != "verbose"]
+        if extra:
+            raise NotImplementedError("AttentionPairBias.forward: unsupported keyword(s) %s" % ", ".join(sorted(extra)))
         a = self.attn
         b, n, _ = single_repr.shape
         h, d = a.heads, a.dim_head

@@ -126,7 +126,7 @@ class OuterProductMean(nn.Module):
         if mask is not None:
             pos = mask.to(torch.float32)[:, None, :, None]                                   # [b, 1, n, 1]
             fa, fb = fa * pos, pos
-        a = a * fa.to(dtype)
+        a = (a.float() * fa).to(dtype)             # one rounding: 1 / rows is not a 16-bit number
         if fb is not None:
             b_ = b_ * fb.to(dtype)
         # outer[(i d), (j e)] = sum_s a[s, i, d] b[s, j, e]: one GEMM per batch element with the contraction axis

@@ -156,7 +156,8 @@ class FusedTransition(nn.Module):
         if self._fused_ln_swiglu and add_residual and input.is_cuda:
             ln = self.ff[0]
             dtype = torch.bfloat16 if torch.is_autocast_enabled() else input.dtype
-            if fused_shape_supported(ln.K, ln.N, dtype, _lib.MF_ACT_SWIGLU):
+            # (an fp32 stream under autocast keeps its separate fp32 add, as the reference's `x + f(x)` promotes)
+            if input.dtype == dtype and fused_shape_supported(ln.K, ln.N, dtype, _lib.MF_ACT_SWIGLU):
                 return _TransitionResidualFunction.apply(input, ln.WEIGHT, ln.BIAS, ln.linear_weight, self.ff[2].weight)
         if self._fused_ln_swiglu:
             # LayerNorm -> Linear -> SwiGLU in one kernel, then the output projection

@@ -278,7 +278,8 @@ class PreLayerNormTriangleAttention(nn.Module):
             raise ValueError("unsupported shape for the fused block: dim=%d heads=%d dim_head=%d" %
                              (dim, attn.heads, attn.dim_head))
         drops = fn.dropout.training and fn.dropout.dropout.p > 0.0
-        fused_sum = add_residual and not drops
+        # an fp32 stream under autocast keeps its separate fp32 add (megafold.py:744-745 promotes)
+        fused_sum = add_residual and not drops and pairwise_repr.dtype == dtype
         out = TriangleAttentionFunction.apply(pairwise_repr, mask, self.norm.weight, self.norm.bias, attn.to_q.weight,
                                               attn.to_q.bias, attn.to_kv.weight, attn.to_gates.weight,
                                               attn.to_gates.bias, fn.to_attn_bias[0].weight, attn.to_out.weight,

@@ -183,7 +183,9 @@ class TriangleMultiplication(nn.Module):
             raise ValueError("unsupported shape for the fused block: dim=%d dim_hidden=%d" % (dim, dh))
         c, o = self.combined, self.to_out[0]
         drop = self.to_out[1]
-        fused_sum = add_residual and not (drop.training and drop.dropout.p > 0.0)
+        # the fused sum adds in the compute dtype: under autocast an fp32 residual stream stays fp32 (x + block(x)
+        # promotes, as in the reference, megafold.py:742-743), so it takes the separate add
+        fused_sum = add_residual and not (drop.training and drop.dropout.p > 0.0) and x.dtype == dtype
         out = TriangleMultiplicationFunction.apply(x, mask, c.WEIGHT, c.BIAS, c.linear_weight, c.linear_bias,
                                                    o.WEIGHT, o.BIAS, o.linear_weight, self.mix == "incoming", fused_sum)
         if fused_sum:

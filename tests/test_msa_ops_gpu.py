@@ -131,6 +131,35 @@ def test_outer_product_mean_parity(b, s, n, dm, dh, dp, use_mask, use_msa_mask, 
         close(name, p.grad, want_dp[name], param_grad_tol(dtype, rows, want_dp[name]))
 
 
+def test_outer_product_mean_at_the_msa_module_size():
+    """[1, 128, 384, 64] MSA in bf16, hidden 32, last 38 positions and three MSA rows masked, against the oracle in fp32
+    on the CPU; 125 kept rows (not a power of two), so a doubly rounded 1 / rows would show in the relative RMS error."""
+    from conftest import rel_rms
+    b, s, n, dm, dh, dp, dtype = 1, 128, 384, 64, 32, 128, torch.bfloat16
+    torch.set_num_threads(16)
+    m = randomise(OuterProductMean(dim_msa=dm, dim_pairwise=dp, dim_hidden=dh), dtype, seed=n)
+    g = torch.Generator().manual_seed(300 + n)
+    msa = torch.randn(b, s, n, dm, generator=g).to(dtype)
+    dout = torch.randn(b, n, n, dp, generator=g).to(dtype)
+    mask = key_mask(b, n, 38)
+    msa_mask = torch.ones(b, s, dtype=torch.bool)
+    msa_mask[:, s - 2:] = False
+    msa_mask[0, 0] = False
+    params = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    want_out, want_dm, want_dp = om.outer_product_mean_forward_backward(msa, params, dout, mask, msa_mask, dtype=torch.float32)
+    m = m.cuda()
+    mg = msa.cuda().requires_grad_(True)
+    out = m(mg, mask=mask.cuda(), msa_mask=msa_mask.cuda())
+    out.backward(dout.cuda())
+    close("out", out, want_out, tol_for(dtype))
+    assert rel_rms(out, want_out) < 4e-3
+    close("dmsa", mg.grad, want_dm, param_grad_tol(dtype, n, want_dm))
+    assert rel_rms(mg.grad, want_dm) < 1e-2
+    for name, p in m.named_parameters():
+        rows = b * n * n if name.startswith("to_pairwise_repr") else b * s * n
+        close(name, p.grad, want_dp[name], param_grad_tol(dtype, rows, want_dp[name]))
+
+
 def test_msa_modules_under_autocast_with_fp32_master_weights():
     """fp32 parameters and inputs under bf16 autocast: bf16 outputs, fp32 gradients for inputs and parameters, values within
     the 16-bit bar of the oracle; dropout of the averaging module zeroes whole rows in training mode only."""

@@ -121,3 +121,42 @@ def test_add_residual_with_active_dropout_falls_back_to_the_separate_sum():
     torch.manual_seed(3)
     b = blk(x) + x
     assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["tri_mult_outgoing", "tri_attn_ending", "pairwise_transition", "block"])
+def test_fp32_residual_stream_under_autocast_stays_fp32(kind):
+    """bf16 autocast with fp32 parameters and an fp32 pair tensor (the reference's bf16-mixed setup): `x + block(x)`
+    promotes to fp32 there (megafold.py:742-747), so add_residual must return fp32 in training and in evaluation
+    mode, hand back an fp32 input gradient, and agree with the separate sum bit for bit (it IS the separate sum)."""
+    n = 24
+    g = torch.Generator().manual_seed(5)
+    full = PairwiseBlock(dropout_row_prob=0.0, dropout_col_prob=0.0).cuda()
+    blk = full if kind == "block" else getattr(full, kind)
+    with torch.no_grad():
+        for p in blk.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.3)
+    x = torch.randn(1, n, n, 128, generator=g).cuda()
+    mask = torch.ones(1, n, dtype=torch.bool, device="cuda")
+    mask[:, n - 3:] = False
+
+    def call(xin, fused):
+        if kind == "block":
+            return blk(pairwise_repr=xin, mask=mask)
+        kw = {} if kind == "pairwise_transition" else {"mask": mask}
+        return blk(xin, add_residual=True, **kw) if fused else blk(xin, **kw) + xin
+
+    for training in (True, False):
+        blk.train(training)
+        xg = x.clone().requires_grad_()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = call(xg, True)
+        assert y.dtype == torch.float32, (kind, training, y.dtype)
+        y.float().square().mean().backward()
+        assert xg.grad.dtype == torch.float32 and torch.isfinite(xg.grad).all()
+        if kind != "block":
+            x2 = x.clone().requires_grad_()
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                y2 = call(x2, False)
+            y2.float().square().mean().backward()
+            assert torch.equal(y, y2) and torch.equal(xg.grad, x2.grad)

@@ -20,10 +20,16 @@ def _both(shape, dtype, seed):
     got_o = torch.full_like(want_o, float("nan"))
     got_lse = torch.full_like(want_lse, float("nan"))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # nothing may come from the caching allocator (not even a transient block that is freed again: the running
+    # counts of allocations and segments must not move) nor from the driver (free device memory must not move)
+    stats = torch.cuda.memory_stats()
+    before = (torch.cuda.memory_allocated(), stats["allocation.all.allocated"], stats["segment.all.allocated"])
+    free_before = torch.cuda.mem_get_info()[0]
     ev.evoattention_forward_noalloc(inp["q"], inp["k"], inp["v"], inp["mask"], inp["bias"], got_o, got_lse)
-    assert torch.cuda.memory_allocated() == before          # nothing came from the caching allocator either
     torch.cuda.synchronize()
+    stats = torch.cuda.memory_stats()
+    assert (torch.cuda.memory_allocated(), stats["allocation.all.allocated"], stats["segment.all.allocated"]) == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return (got_o, got_lse), (want_o, want_lse)
 
 
