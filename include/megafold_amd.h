@@ -64,8 +64,9 @@ const char* mf_last_error(void);
  *           keep-mask: true -> 0, false -> -inf.
  *   lse   : [B, N, H, S] fp32, written by fwd, read by bwd.
  *   dbias : [B, H, S, S] fp32 contiguous, written by bwd; NULL = the bias needs no gradient.
- * Supported: D multiple of 8, D <= 64; dtype f32 / f16 / bf16; strides of q..dv multiples of
- * 16 bytes; pointers 16-byte aligned.
+ * Supported: D multiple of 8, D <= 64; S <= MF_EVOATTN_MAX_S; dtype f32 / f16 / bf16; strides of
+ * q..dv multiples of 16 bytes; pointers 16-byte aligned.  Anything else: MF_ERR_SHAPE / _DTYPE / _STRIDE with a
+ * message (mf_last_error), before anything is launched.
  * A query row whose keys are all masked with -inf yields o = 0, lse = -inf and zero gradients.
  * ---------------------------------------------------------------------------------------------- */
 /* Backward phases.  MF_EVO_BWD_PREP copies the pair bias into the workspace (scaled, padded, fp32);
@@ -75,6 +76,7 @@ const char* mf_last_error(void);
  * all of them (DBIAS only when dbias != NULL).
  * The workspace size depends on the shape, on whether dbias is requested and on the number of compute units of
  * the CURRENT device: query it with the arguments of the call and with the device of the call current. */
+#define MF_EVOATTN_MAX_S 16384
 #define MF_EVO_BWD_DQKV 1
 #define MF_EVO_BWD_DBIAS 2
 #define MF_EVO_BWD_PREP 4

@@ -63,6 +63,8 @@ int check_common(const mf_evoattn_args* a) {
   if (a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0)
     return fail(MF_ERR_SHAPE, "B, N, S, H, D must be positive (got %d %d %d %d %d)", a->B, a->N, a->S, a->H, a->D);
   if (a->D % 8 != 0 || a->D > 64) return fail(MF_ERR_SHAPE, "D=%d unsupported: need a multiple of 8, at most 64", a->D);
+  // the forward keeps the mask values of a row (4 S bytes) in LDS next to its tiles
+  if (a->S > MF_EVOATTN_MAX_S) return fail(MF_ERR_SHAPE, "S=%d unsupported: at most %d", a->S, MF_EVOATTN_MAX_S);
   if (a->dtype != MF_DTYPE_F32 && a->dtype != MF_DTYPE_F16 && a->dtype != MF_DTYPE_BF16)
     return fail(MF_ERR_DTYPE, "dtype %d unsupported for q/k/v", a->dtype);
   if (a->bias_dtype != MF_DTYPE_F32 && a->bias_dtype != MF_DTYPE_F16 && a->bias_dtype != MF_DTYPE_BF16)

@@ -696,6 +696,7 @@ template <typename T> static hipError_t launch_dqkv_rk(const EvoParams& p, hipSt
   int best_nw = 4;
   long long best_cost = -1;
   for (int nw = 4; nw <= 8; ++nw) {
+    if (nw > 4 && RkLayout<T>::smem(nw, NT) > 160 * 1024) continue;   // four wavefronts fit: the caller has checked
     const int chunks = (NT + nw - 1) / nw;
     const int resident = nw * (8 / nw);
     const long long cost = ((long long)chunks * nw * 840 / resident) * 64 + chunks;
@@ -1127,14 +1128,12 @@ __global__ void __launch_bounds__(256) dbias_reduce_kernel(const float* part, fl
 // Key tiles per wavefront patch: limited by the registers the patch and its bias seed occupy.
 static int dbias_tr(int dtype, int D) { return (dtype == MF_F32 || D > 32) ? 1 : 2; }
 
+// Compute units of the CURRENT device, asked on every call: a process may drive several devices, and the
+// answer decides grids and workspace sizes (256 when no device can be queried, e.g. without a GPU).
 static int dbias_num_cu() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0, n = 0;
-    cached = (hipGetDevice(&dev) == hipSuccess &&
-              hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
-  }
-  return cached;
+  int dev = 0, n = 0;
+  return (hipGetDevice(&dev) == hipSuccess &&
+          hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
 }
 
 // Number of chunks the N rows are split into.  Work-groups of one (b, h, chunk) group are placed on

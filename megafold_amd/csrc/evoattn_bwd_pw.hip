@@ -21,7 +21,9 @@
 //    scores and dP are ordinary vector registers, where the vector ALU reads them without copies.
 //  * With four wavefronts of TPW = 3 tiles a work-group covers 384 keys: at S <= 384 every query tile is
 //    read once and dQ is written once.  Longer sequences run in passes of 4 * TPW key tiles; the running
-//    dQ then stays in an fp32 LDS array until the last pass (no rounding between passes).
+//    dQ then stays, in fp32 (no rounding between passes), in an array of the work-group's own in global memory
+//    (EvoParams::dq_scratch: one [ceil(S/32) * 32, 32] array per work-group, so its size, and with it the
+//    backward's workspace, follows the compute-unit count of the device the launch runs on).
 //  * One work-group per compute unit, looping over its share of the (b, n, h) problems: all heads of a
 //    row n are handled by the same XCD at the same time, because two heads share every 128-byte line of
 //    Q, K, V, dO.

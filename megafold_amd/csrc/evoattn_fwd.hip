@@ -334,11 +334,16 @@ __global__ void __launch_bounds__(256, WPE) evo_fwd_kernel(const EvoParams p, co
   }
 }
 
-template <typename T, int DP, int R, int WPE> static hipError_t launch_fwd_t(const EvoParams& p, hipStream_t stream) {
+// LDS of a work-group with R rows: K / V tiles of the rows, double buffered, and the rows' mask values
+template <typename T, int DP> static size_t fwd_smem(int R, int NT) {
   using L = FwdLayout<T, DP>;
+  return (size_t)4 * R * 32 * L::KSTR * sizeof(T) + ((size_t)R * NT * 32 + 4) * 4;
+}
+
+template <typename T, int DP, int R, int WPE> static hipError_t launch_fwd_t(const EvoParams& p, hipStream_t stream) {
   const int NT = (p.S + 31) / 32;
-  const size_t smem = (size_t)4 * R * 32 * L::KSTR * sizeof(T) + ((size_t)R * NT * 32 + 4) * 4;
-  if (smem > 160 * 1024) return hipErrorInvalidValue;
+  const size_t smem = fwd_smem<T, DP>(R, NT);
+  if (smem > 160 * 1024) return hipErrorInvalidValue;   // not reached: launch_fwd_d lowers R until the rows fit
   const int QB = (p.S + 127) / 128;
   const int NG = (p.N + R - 1) / R;
   const long long blocks = (long long)round_up(p.B * NG, 8) * p.H * QB;
@@ -353,16 +358,6 @@ template <typename T, int DP, int R, int WPE> static hipError_t launch_fwd_t(con
   return hipGetLastError();
 }
 
-static int fwd_num_cu() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0, n = 0;
-    cached = (hipGetDevice(&dev) == hipSuccess &&
-              hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
-  }
-  return cached;
-}
-
 // Rows n per work-group (R).  More rows share one pair-bias tile, but the grid runs in whole rounds of
 // resident work-groups (3 per compute unit for R = 2, 2 for R = 3 and 4), and a stage costs about
 // 7 + R units of time, so the best R is the one with the smallest rounds * (7 + R) (fitted to
@@ -370,17 +365,22 @@ static int fwd_num_cu() {
 template <typename T> static hipError_t launch_fwd_d(const EvoParams& p, hipStream_t stream) {
   constexpr bool wide = sizeof(T) == 4;
   const long long QB = (p.S + 127) / 128;
+  const int num_cu = evo_num_cu();
   int rows = 4;
   double best = -1.0;
   for (int r = 2; r <= 4; ++r) {
     const long long wgs = (long long)round_up(p.B * ((p.N + r - 1) / r), 8) * p.H * QB;
-    const long long slots = (long long)(r == 2 ? 3 : 2) * fwd_num_cu();
+    const long long slots = (long long)(r == 2 ? 3 : 2) * num_cu;
     const double cost = (double)((wgs + slots - 1) / slots) * (7.0 + r);
     if (best < 0.0 || cost < best) { best = cost; rows = r; }
   }
   const long long groups1 = (long long)p.B * p.N * p.H * QB;
   if (groups1 < 2048) rows = rows > 2 ? 2 : rows;   // small problems: keep enough work-groups
   if (groups1 < 1024 || p.N == 1) rows = 1;
+  // very long sequences: the rows' mask values (4 R S bytes) must fit the LDS next to the tiles; one row always
+  // does for the sequence lengths the C ABI admits
+  const int NT = (p.S + 31) / 32;
+  while (rows > 1 && (p.D <= 32 ? fwd_smem<T, 32>(rows, NT) : fwd_smem<T, 64>(rows, NT)) > 160 * 1024) --rows;
   if constexpr (wide) {
     if (p.D <= 32) return rows >= 2 ? launch_fwd_t<T, 32, 2, 2>(p, stream) : launch_fwd_t<T, 32, 1, 2>(p, stream);
     if (p.D <= 64) return launch_fwd_t<T, 64, 1, 2>(p, stream);

@@ -6,7 +6,7 @@ form only:
 * ``AttentionPairBias.forward``  megafold/model/megafold.py:537-591   ``attn_bias = to_attn_bias(pairwise) + attn_bias``
   with ``to_attn_bias = LayernormLinear(dim_pairwise, heads, no bias) ; "b ... h -> b h ..."`` (megafold.py:530-534),
   then ``attn(single_repr, attn_bias=..., mask=...)``
-* ``LayernormLinear``            megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:1017-1047
+* ``LayernormLinear``            megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:498-545
   ``LayerNorm(x; WEIGHT, BIAS, eps 1e-5) @ linear_weight`` with ``linear_weight`` stored ``[K, N]``
 * ``Attention.forward``          megafold/model/attention.py:158-209  q = to_q(x); k, v = to_kv(x).chunk(2);
   split heads ``"b n (h d) -> b h n d"``; attend; merge heads; ``out * sigmoid(to_gates(x))``; ``to_out``

@@ -9,7 +9,7 @@ One tensor expression per reference statement:
 * ``OuterProductMean.forward``          megafold/model/megafold.py:764-824 (Algorithm 9)
   ``a, b = LayernormLinear(msa).chunk(2)``; MSA-row mask on both; ``einsum "b s i d, b s j e -> b i j d e"``;
   divide by the number of kept MSA rows (clamped at eps) or by ``s``; flatten ``(d e)``; pair mask; ``Linear``
-* ``LayernormLinear``  megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:1017-1047
+* ``LayernormLinear``  megafold/model/FusedLayernormLinear/fused_layernorm_linear.py:498-545
   ``LayerNorm(x; WEIGHT, BIAS, eps 1e-5) @ linear_weight`` with ``linear_weight`` stored ``[K, N]``
 
 Masked keys get -inf where the reference fills with the most negative finite value (megafold.py:886-888): the

@@ -72,6 +72,7 @@ def _evo_args():
     (lambda a: setattr(a, "D", 12), -2, "D=12"),
     (lambda a: setattr(a, "D", 128), -2, "D=128"),
     (lambda a: setattr(a, "S", 0), -2, "positive"),
+    (lambda a: setattr(a, "S", 16385), -2, "at most 16384"),
     (lambda a: setattr(a, "dtype", 7), -3, "dtype 7"),
     (lambda a: setattr(a, "mask_dtype", 9), -3, "mask_dtype"),
     (lambda a: setattr(a, "k_stride", _lib.I64x4(8192, 4096, 63, 32)), -4, "k stride[2]=63"),

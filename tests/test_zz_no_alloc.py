@@ -35,6 +35,12 @@ def _both(shape, dtype, seed):
 
 def test_noalloc_matches_workspace_form_twice():
     print("noalloc big then small", flush=True)
+    # the entry point's first call on a device is its set-up: the runtime loads the library's device image, which
+    # is when the fixed scratch array gets its memory; the calls after it must leave the device's free memory alone
+    tiny = {k: v.cuda() for k, v in workloads.evoattention_inputs(1, 1, 32, 1, 8, 0, dtype=torch.bfloat16, seed=1).items()}
+    ev.evoattention_forward_noalloc(tiny["q"], tiny["k"], tiny["v"], tiny["mask"], tiny["bias"],
+                                    torch.empty_like(tiny["q"]), torch.empty(1, 1, 1, 32, device="cuda"))
+    torch.cuda.synchronize()
     for shape, dtype, seed in (((1, 6, 200, 4, 32, 17), torch.bfloat16, 5), ((2, 2, 45, 2, 16, 3), torch.float32, 6)):
         got, want = _both(shape, dtype, seed)
         for g, w in zip(got, want):
