@@ -255,6 +255,48 @@ int mf_channels_last_to_first(const mf_trimul_args* a);
 int mf_channels_first_to_last(const mf_trimul_args* a);
 
 /* ------------------------------------------------------------------------------------------------
+ * MSA pair-weighted averaging (Algorithm 10), the contraction part of MSAPairWeightedAveraging.forward
+ * (megafold/model/megafold.py:868-902): the weights  w[b,h,i,:] = softmax_j(logits[b,i,j,h] + mask[b,j])  do not
+ * depend on the MSA row, so they are formed once and applied to every row:
+ *   y[b,s,i,h,:] = (sum_j w[b,h,i,j] x[b,s,j,h,:]) * sigmoid(g[b,s,i,h,:])
+ * 16-bit element types, H = 8 heads of D = 32 channels.
+ *   logits, dlogits : rows [B*N*N] of H elements, ld_* elements apart (a multiple of 8)
+ *   mask            : [B, N] bytes, non-zero = keep, or NULL; a row whose keys are all masked gets zero weights
+ *   w               : [B, H, NP, NP], NP = N rounded up to 32, zero outside [N, N]
+ *   x, g, y, dy     : rows [B*S*N] of H*D elements (channels of head h at 32 h), ld* elements apart (multiples
+ *                     of 8, >= 256): column slices of wider matrices are fine
+ *   dw_part         : [n_chunks, B, H, NP, NP] fp32, n_chunks = mf_pwa_dw_chunks(args)
+ * mf_pwa_softmax_fwd   logits, mask -> w
+ * mf_pwa_apply         w, x (, g) -> y; N <= 384.  With the transposed weights as w and dy as x it computes
+ *                      dx[b,s,j,h,:] = sum_i w[b,h,i,j] dy[b,s,i,h,:]
+ * mf_pwa_dw            dy, x -> dw_part: partial sums over chunks of the MSA rows of
+ *                      dw[b,h,i,j] = sum_{s,d} dy[b,s,i,h,d] x[b,s,j,h,d]
+ * mf_pwa_softmax_bwd   w, dw_part -> dlogits = w * (dw - sum_j w dw), dw = the sum of the partial buffers
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct {
+  int32_t B, S, N, H, D;
+  int32_t dtype;
+  int32_t n_chunks;
+  int32_t reserved0;
+  const void* logits; int64_t ld_logits;
+  const void* mask;
+  void* w;
+  const void* x;  int64_t ldx;
+  const void* g;  int64_t ldg;
+  void* y;        int64_t ldy;
+  const void* dy; int64_t lddy;
+  float* dw_part;
+  void* dlogits;  int64_t ld_dlogits;
+  void* stream;
+} mf_pwa_args;
+
+int mf_pwa_softmax_fwd(const mf_pwa_args* a);
+int mf_pwa_apply(const mf_pwa_args* a);
+int mf_pwa_dw_chunks(const mf_pwa_args* a);
+int mf_pwa_dw(const mf_pwa_args* a);
+int mf_pwa_softmax_bwd(const mf_pwa_args* a);
+
+/* ------------------------------------------------------------------------------------------------
  * y[a][c][b][:] = x[a][b][c][:] for contiguous arrays of rows of `row_bytes` bytes (a multiple of 16, at most
  * 256): the layout move between the [(i d), (j e)] result of OuterProductMean's contraction and the
  * "b i j (d e)" rows its projection reads (megafold/model/megafold.py:795, 807, 812), and the inverse move for

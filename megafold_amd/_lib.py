@@ -69,6 +69,17 @@ class TriMulArgs(C.Structure):
     ]
 
 
+class PwaArgs(C.Structure):
+    _fields_ = [
+        ("B", C.c_int32), ("S", C.c_int32), ("N", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32), ("n_chunks", C.c_int32), ("reserved0", C.c_int32),
+        ("logits", C.c_void_p), ("ld_logits", C.c_int64), ("mask", C.c_void_p), ("w", C.c_void_p),
+        ("x", C.c_void_p), ("ldx", C.c_int64), ("g", C.c_void_p), ("ldg", C.c_int64),
+        ("y", C.c_void_p), ("ldy", C.c_int64), ("dy", C.c_void_p), ("lddy", C.c_int64),
+        ("dw_part", C.c_void_p), ("dlogits", C.c_void_p), ("ld_dlogits", C.c_int64), ("stream", C.c_void_p),
+    ]
+
+
 # every symbol include/megafold_amd.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "mf_version": (C.c_int, []),
@@ -88,6 +99,11 @@ SYMBOLS = {
     "mf_swiglu_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]),
     "mf_sigmoid_gate_fwd": (C.c_int, [C.POINTER(GateArgs)]),
     "mf_sigmoid_gate_bwd": (C.c_int, [C.POINTER(GateArgs)]),
+    "mf_pwa_softmax_fwd": (C.c_int, [C.POINTER(PwaArgs)]),
+    "mf_pwa_apply": (C.c_int, [C.POINTER(PwaArgs)]),
+    "mf_pwa_dw_chunks": (C.c_int, [C.POINTER(PwaArgs)]),
+    "mf_pwa_dw": (C.c_int, [C.POINTER(PwaArgs)]),
+    "mf_pwa_softmax_bwd": (C.c_int, [C.POINTER(PwaArgs)]),
     "mf_trimul_pack_fwd": (C.c_int, [C.POINTER(TriMulArgs)]),
     "mf_trimul_pack_bwd": (C.c_int, [C.POINTER(TriMulArgs)]),
     "mf_channels_last_to_first": (C.c_int, [C.POINTER(TriMulArgs)]),

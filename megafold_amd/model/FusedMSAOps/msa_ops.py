@@ -30,13 +30,93 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+import ctypes as C
+
+from ... import _lib
 from ..FusedEvoAttention.evoattention import TritonEvoformer
 from ..FusedLayernormLinear.fused_layernorm_linear import LayernormLinear
 from ..FusedTriangleAttention.triangle_attention import Dropout
+from ..FusedTriangleAttention.triangle_attention import sigmoid_gate_backward
 from ..gate import sigmoid_gate
 from ..linear import linear_no_bias
 
 __all__ = ["MSAPairWeightedAveraging", "OuterProductMean"]
+
+
+def _pwa_args(b, s, n, h, d, dtype, device):
+    a = _lib.PwaArgs()
+    a.B, a.S, a.N, a.H, a.D = b, s, n, h, d
+    a.dtype = _lib.dtype_code(dtype)
+    a.stream = torch.cuda.current_stream(device).cuda_stream
+    return a
+
+
+def _pwa_apply(W, X, G, dims, out=None):
+    """``out[(b s i), (h d)] = sum_j W[b, h, i, j] X[(b s j), (h d)]`` (times ``sigmoid(G)`` if given) through
+    ``mf_pwa_apply``; X, G, out: matrices of rows with unit stride along the columns (column slices are fine)."""
+    b, s, n, h, d = dims
+    if out is None:
+        out = torch.empty((b * s * n, h * d), dtype=X.dtype, device=X.device)
+    a = _pwa_args(b, s, n, h, d, X.dtype, X.device)
+    a.w = W.data_ptr()
+    a.x, a.ldx = X.data_ptr(), X.stride(0)
+    if G is not None:
+        a.g, a.ldg = G.data_ptr(), G.stride(0)
+    a.y, a.ldy = out.data_ptr(), out.stride(0)
+    _lib.check(_lib.lib().mf_pwa_apply(C.byref(a)), "mf_pwa_apply")
+    return out
+
+
+class PairWeightedAverageFunction(torch.autograd.Function):
+    """``A[(b s i), (h d)] = (sum_j softmax_j(logits[b, i, j, h] + mask[b, j]) V[(b s j), (h d)]) * sigmoid(G)`` with
+    V | G the two column halves of ``vg`` (megafold.py:884-893): the softmax once per (b, h, i), the averaging and
+    the gate in one kernel with the weight rows resident in registers across the MSA rows.  Backward: the gate's
+    derivative on the recomputed averages, dV through the same kernel on the transposed weights, the weights'
+    gradient as a contraction over (MSA row, channel) with the softmax backward behind it."""
+
+    @staticmethod
+    def forward(ctx, logits, vg, mask, dims):
+        b, s, n, h, d = dims
+        inner = h * d
+        NP = (n + 31) // 32 * 32
+        with torch.cuda.device(vg.device):
+            W = torch.empty((b, h, NP, NP), dtype=vg.dtype, device=vg.device)
+            a = _pwa_args(b, s, n, h, d, vg.dtype, vg.device)
+            a.logits, a.ld_logits = logits.data_ptr(), logits.stride(0)
+            a.mask = mask.data_ptr() if mask is not None else None
+            a.w = W.data_ptr()
+            _lib.check(_lib.lib().mf_pwa_softmax_fwd(C.byref(a)), "mf_pwa_softmax_fwd")
+            A = _pwa_apply(W, vg[:, :inner], vg[:, inner:], dims)
+        ctx.save_for_backward(W, vg, logits)
+        ctx.dims = dims
+        return A
+
+    @staticmethod
+    def backward(ctx, dA):
+        W, vg, logits = ctx.saved_tensors
+        b, s, n, h, d = dims = ctx.dims
+        inner = h * d
+        lib = _lib.lib()
+        with torch.cuda.device(vg.device):
+            dA = dA.to(vg.dtype)
+            dA = dA if dA.stride(1) == 1 else dA.contiguous()
+            V, G = vg[:, :inner], vg[:, inner:]
+            O = _pwa_apply(W, V, None, dims)                               # the averages before the gate, recomputed
+            dvg = torch.empty_like(vg)
+            dO, _ = sigmoid_gate_backward(dA, O, G, dvg[:, inner:], need_product=False)
+            _pwa_apply(W.transpose(-1, -2).contiguous(), dO, None, dims, out=dvg[:, :inner])    # dV
+            a = _pwa_args(b, s, n, h, d, vg.dtype, vg.device)
+            a.w = W.data_ptr()
+            a.x, a.ldx = V.data_ptr(), V.stride(0)
+            a.dy, a.lddy = dO.data_ptr(), dO.stride(0)
+            a.n_chunks = lib.mf_pwa_dw_chunks(C.byref(a))
+            part = torch.empty((a.n_chunks,) + tuple(W.shape), dtype=torch.float32, device=vg.device)
+            a.dw_part = part.data_ptr()
+            _lib.check(lib.mf_pwa_dw(C.byref(a)), "mf_pwa_dw")
+            dlogits = torch.empty_like(logits)
+            a.dlogits, a.ld_dlogits = dlogits.data_ptr(), dlogits.stride(0)
+            _lib.check(lib.mf_pwa_softmax_bwd(C.byref(a)), "mf_pwa_softmax_bwd")
+        return dlogits, dvg, None, None
 
 
 class MSAPairWeightedAveraging(nn.Module):
@@ -58,15 +138,25 @@ class MSAPairWeightedAveraging(nn.Module):
         h, d = self.heads, self.dim_head
         inner = h * d
         vg = self.msa_to_values_and_gates(msa)                                   # [b, s, n, (gv h d)]
-        V = vg[..., :inner].unflatten(-1, (h, d))                                # view [b, s, n, h, d]
-        bias = self.pairwise_repr_to_attn(pairwise_repr).permute(0, 3, 1, 2).unsqueeze(1)   # view [b, 1, h, i, j]
-        if mask is not None:
-            res_mask = mask.view(b, 1, 1, 1, n)                                  # keep-mask, shared by all rows s
+        logits = self.pairwise_repr_to_attn(pairwise_repr)                       # [b, i, j, h]
+        if (h == 8 and d == 32 and n <= 384 and vg.dtype in (torch.float16, torch.bfloat16) and logits.dtype == vg.dtype
+                and vg.is_contiguous() and logits.is_contiguous()):
+            # the dedicated kernels: softmax once per (b, h, i), then the averaging with the gate in its epilogue
+            keep = mask.to(torch.uint8).contiguous() if mask is not None else None
+            A = PairWeightedAverageFunction.apply(logits.view(b * n * n, h), vg.view(b * s * n, 2 * inner), keep,
+                                                  (b, s, n, h, d))
         else:
-            res_mask = torch.zeros(b, 1, 1, 1, n, dtype=torch.float32, device=msa.device)
-        zero = torch.zeros(d, dtype=vg.dtype, device=vg.device).expand(b, s, n, h, d)   # queries = keys = 0
-        O = TritonEvoformer(zero, zero, V, res_mask, bias)                        # softmax(bias) @ values
-        A = sigmoid_gate(O.reshape(b * s * n, inner), vg.view(b * s * n, 2 * inner)[:, inner:])
+            # other shapes: the pair-biased attention operator with zero queries and keys and the MSA rows as
+            # its row batch (the bias is shared by all rows), then the gate
+            V = vg[..., :inner].unflatten(-1, (h, d))                            # view [b, s, n, h, d]
+            bias = logits.permute(0, 3, 1, 2).unsqueeze(1)                       # view [b, 1, h, i, j]
+            if mask is not None:
+                res_mask = mask.view(b, 1, 1, 1, n)                              # keep-mask, shared by all rows s
+            else:
+                res_mask = torch.zeros(b, 1, 1, 1, n, dtype=torch.float32, device=msa.device)
+            zero = torch.zeros(d, dtype=vg.dtype, device=vg.device).expand(b, s, n, h, d)   # queries = keys = 0
+            O = TritonEvoformer(zero, zero, V, res_mask, bias)                    # softmax(bias) @ values
+            A = sigmoid_gate(O.reshape(b * s * n, inner), vg.view(b * s * n, 2 * inner)[:, inner:])
         out = linear_no_bias(A.view(b, s, n, inner), self.to_out[1].weight)
         return self.to_out[2](out)
 
