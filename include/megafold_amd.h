@@ -297,6 +297,19 @@ int mf_pwa_dw(const mf_pwa_args* a);
 int mf_pwa_softmax_bwd(const mf_pwa_args* a);
 
 /* ------------------------------------------------------------------------------------------------
+ * Outer product mean (Algorithm 9), the contraction part of OuterProductMean.forward
+ * (megafold/model/megafold.py:795-823) in one kernel, without the [n, n, dh*dh] tensor:
+ *   out[b,i,j,:] = sum_{d,e} w[:, e*32 + d] * (sum_s a[b, i*32 + d, s] * b[b, j*32 + e, s]) + bias
+ *   a, b : [B, n*32, 128] (hidden dimension 32; the MSA rows s along the contiguous axis, zero padded to 128;
+ *          masks and the division by the number of rows already applied)
+ *   w    : [128, 1024]: the projection weight with its two hidden indices exchanged (column e*32 + d holds
+ *          the reference's column d*32 + e); bias : [128] or NULL; out : [B, n, n, 128]
+ * 16-bit element types.
+ * ---------------------------------------------------------------------------------------------- */
+int mf_opm_fused_fwd(const void* a, const void* b, const void* w, const void* bias, void* out, int32_t B, int32_t n,
+                     int32_t dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * y[a][c][b][:] = x[a][b][c][:] for contiguous arrays of rows of `row_bytes` bytes (a multiple of 16, at most
  * 256): the layout move between the [(i d), (j e)] result of OuterProductMean's contraction and the
  * "b i j (d e)" rows its projection reads (megafold/model/megafold.py:795, 807, 812), and the inverse move for

@@ -1,0 +1,207 @@
+// Outer product mean (Algorithm 9 of AlphaFold 3), the contraction part of the reference's
+// OuterProductMean.forward (megafold/model/megafold.py:795-823):
+//
+//     outer[b,i,j,d,e] = sum_s a[b,s,i,d] b[b,s,j,e]                 megafold.py:795, 807   (a, b already masked / scaled)
+//     out[b,i,j,:]     = W[:, (d e)] . outer[b,i,j,(d e)] + bias      megafold.py:812, 823
+//
+// in ONE kernel: the [n, n, dh * dh] tensor (302 MB at n = 384, dh = 32) never exists.  With the operands as
+// matrices A[(i d), s] and B[(j e), s] (s contiguous), the 32 x 32 accumulator tile of rows (i, .) and columns
+// (j, .) of A B^T IS the outer block of the position pair (i, j); it is rounded to 16 bits, laid into LDS as one
+// row of 1024 values per pair, and 32 such rows are then multiplied with the projection weight, which every
+// wavefront keeps in registers (a quarter of the output channels times half of the 1024 products each) for all
+// the pair tiles its work-group walks over.
+//   work-group  = eight wavefronts, persistent over a contiguous run of pair tiles (8 rows i x 4 columns j)
+//   stage 1     wavefront w: the four outer blocks (i0 + w, j0 .. j0 + 3); A rows from global memory (reloaded
+//               only when i0 changes), B rows of the tile from LDS (direct loads, double buffered)
+//   stage 2     wavefront (channel tile ct, half kh): out[32 pairs, 32 channels] over its 512 products; the two
+//               halves meet in LDS, bias added, 32-byte runs stored
+// 16-bit element types, dh = 32, 128 output channels, s <= 128 (the operands are zero padded to 128 columns).
+#include "../../include/megafold_amd.h"
+#include "capi_common.h"
+#include "common.h"
+
+namespace mf {
+namespace {
+
+struct OpmParams {
+  int B, n, tiles_j, tiles, per_group;
+  const void* a;      // [B, n * 32, 128]
+  const void* b;      // [B, n * 32, 128]
+  const void* w;      // [128, 1024], column e * 32 + d (the reference's weight with d and e exchanged)
+  const void* bias;   // [128] or nullptr
+  void* out;          // [B, n, n, 128]
+};
+
+constexpr int OB_STRIDE = 2048 + 16;            // bytes between pair rows of the outer-block buffer
+constexpr int LDS_B = 0;                        // two B tiles of 128 rows x 256 bytes
+constexpr int LDS_O = 2 * 32768;                // 32 pair rows
+constexpr int LDS_P = LDS_O + 32 * OB_STRIDE;   // partial sums of the second half: [4 channel tiles][64 lanes][16] fp32
+constexpr int LDS_BYTES = LDS_P + 4 * 64 * 16 * 4;
+
+__device__ __forceinline__ void dma16(unsigned voff, const void* sbase, unsigned lds) {
+  asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "{m0}"(lds) : "memory");
+}
+template <int VM> __device__ __forceinline__ void wait_vm() {
+  __builtin_amdgcn_s_waitcnt(((VM & 15) | ((VM >> 4) << 14)) | (7 << 4) | (15 << 8));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(512, 1) opm_fused_kernel(const OpmParams p) {
+  using frag = frag_t<T>;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t512 = threadIdx.x;
+  const int wv = __builtin_amdgcn_readfirstlane(t512 >> 6);
+  const int l = t512 & 63, x = l & 31, g = l >> 5;
+  const int ct = wv & 3, kh = wv >> 2;
+  const int n = p.n;
+
+  const int t_begin = blockIdx.x * p.per_group;
+  const int t_end = min(p.tiles, t_begin + p.per_group);
+  if (t_begin >= t_end) return;
+
+  // ---- the projection weight of this wavefront: A operands of stage 2 (rows = channels, permuted so that an
+  // accumulator holds 16 consecutive channels per lane), 32 steps of 16 products, resident
+  frag wf[32];
+  {
+    const T* wrow = reinterpret_cast<const T*>(p.w) + (int64_t)(ct * 32 + unperm32(x)) * 1024 + kh * 512 + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < 32; ++ks) wf[ks] = ld8<T>(wrow + 16 * ks);
+#pragma unroll
+    for (int ks = 0; ks < 32; ++ks) pin(wf[ks]);
+  }
+  float bias_c[16];
+  {
+    frag b0 = frag_zero<T>(), b1 = frag_zero<T>();
+    if (p.bias) {
+      b0 = ld8<T>(reinterpret_cast<const T*>(p.bias) + ct * 32 + 16 * g);
+      b1 = ld8<T>(reinterpret_cast<const T*>(p.bias) + ct * 32 + 16 * g + 8);
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) { bias_c[r] = (float)b0[r]; bias_c[8 + r] = (float)b1[r]; }
+  }
+
+  // ---- direct loads of a B tile: LDS row r (0..127) = row (j0 * 32 + r) of the operand, 16-byte chunk c of a row
+  // at position c ^ (r & 15) (conflict-free fragment reads)
+  const unsigned lds0 = (unsigned)(unsigned long)((__attribute__((address_space(3))) unsigned char*)smem);
+  auto issue_b = [&](int tile, int buf) {
+    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+    const int j0 = (rem % p.tiles_j) * 4;
+    const char* base = reinterpret_cast<const char*>(p.b) + (int64_t)bb * n * 32 * 256;
+#pragma unroll
+    for (int rd = 0; rd < 4; ++rd) {
+      const int q = rd * 512 + t512, row = q >> 4, pos = q & 15;
+      int grow = j0 * 32 + row;
+      grow = grow < n * 32 ? grow : n * 32 - 1;
+      dma16((unsigned)(grow * 256 + ((pos ^ (row & 15)) << 4)), base, lds0 + LDS_B + buf * 32768 + rd * 8192 + wv * 1024);
+    }
+  };
+
+  unsigned char* Ob = smem + LDS_O;
+  float* Pp = reinterpret_cast<float*>(smem + LDS_P);
+  frag af[8];
+  int cur_i0 = -1, cur_b = -1;
+  issue_b(t_begin, 0);
+  for (int tile = t_begin; tile < t_end; ++tile) {
+    const int buf = (tile - t_begin) & 1;
+    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+    // ---- stage 1: A rows of row i0 + wv (B operands of the product: columns = d, permuted), once per i0
+    if (i0 != cur_i0 || bb != cur_b) {
+      int i = i0 + wv;
+      i = i < n ? i : n - 1;
+      const T* arow = reinterpret_cast<const T*>(p.a) + ((int64_t)bb * n * 32 + i * 32 + unperm32(x)) * 128 + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) af[ks] = ld8<T>(arow + 16 * ks);
+      cur_i0 = i0; cur_b = bb;
+    }
+    wait_vm<0>();                                  // this tile's B rows (and the A rows) have arrived
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();                  // ... for every wavefront; the other B slot and the outer-block
+    asm volatile("" ::: "memory");                 // buffer are free (their readers are past the preceding tile)
+    if (tile + 1 < t_end) issue_b(tile + 1, buf ^ 1);
+    const unsigned char* Bt = smem + LDS_B + buf * 32768;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      f32x16 acc = acc_zero();
+      const int row = jj * 32 + x;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const frag bf = ld8<T>(reinterpret_cast<const T*>(Bt + row * 256 + (((2 * ks + g) ^ (row & 15)) << 4)));
+        acc = mma(af[ks], bf, acc);                // rows = d (16 g + r in register r), columns = e
+      }
+      // pair row (wv * 4 + jj) of the buffer: product index e * 32 + d, 16-byte chunk q at q ^ ((q >> 4) & 3)
+      unsigned char* orow = Ob + (wv * 4 + jj) * OB_STRIDE;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int q = 4 * x + 2 * g + u;
+        st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), acc_half<T>(acc, u));
+      }
+    }
+    barrier_keep_vm<63>();                         // LDS hand-over only: the next B tile keeps travelling
+    // ---- stage 2: out[pair, 32 channels of tile ct] over this wavefront's 512 products
+    f32x16 o = acc_zero();
+#pragma unroll
+    for (int ks = 0; ks < 32; ++ks) {
+      const int q = kh * 64 + 2 * ks + g;
+      const frag of = ld8<T>(reinterpret_cast<const T*>(Ob + x * OB_STRIDE + ((q ^ ((q >> 4) & 3)) << 4)));
+      o = mma(wf[ks], of, o);                      // rows = channels (16 g + r in register r), columns = pairs
+    }
+    if (kh == 1) {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        f32x4 v = {o[4 * c4], o[4 * c4 + 1], o[4 * c4 + 2], o[4 * c4 + 3]};
+        *reinterpret_cast<f32x4*>(Pp + ((ct * 4 + c4) * 64 + l) * 4) = v;
+      }
+    }
+    barrier_keep_vm<63>();                         // LDS hand-over only: the next B tile keeps travelling
+    if (kh == 0) {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(Pp + ((ct * 4 + c4) * 64 + l) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[4 * c4 + e] += v[e] + bias_c[4 * c4 + e];
+      }
+      const int i = i0 + (x >> 2), j = j0 + (x & 3);     // lane x = pair row of the buffer
+      if (i < n && j < n) {
+        T* op = reinterpret_cast<T*>(p.out) + (((int64_t)bb * n + i) * n + j) * 128 + ct * 32 + 16 * g;
+        st8<T>(op, acc_half<T>(o, 0));
+        st8<T>(op + 8, acc_half<T>(o, 1));
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace mf
+
+using namespace mf;
+
+extern "C" int mf_opm_fused_fwd(const void* a, const void* b, const void* w, const void* bias, void* out, int32_t B,
+                                int32_t n, int32_t dtype, void* stream) {
+  clear_error();
+  if (!a || !b || !w || !out) return fail(MF_ERR_NULL, "a, b, w or out is NULL");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(w) || !aligned16(out)) return fail(MF_ERR_ALIGN, "operands must be 16-byte aligned");
+  if (B <= 0 || n <= 0) return fail(MF_ERR_SHAPE, "B, n must be positive (got %d, %d)", B, n);
+  if ((int64_t)n * 32 * 256 >= (1LL << 31)) return fail(MF_ERR_SHAPE, "n=%d too large", n);
+  if (dtype != MF_DTYPE_F16 && dtype != MF_DTYPE_BF16) return fail(MF_ERR_DTYPE, "dtype %d unsupported: f16 / bf16", dtype);
+  OpmParams p{};
+  p.B = B; p.n = n;
+  p.tiles_j = (n + 3) / 4;
+  const int64_t tiles = (int64_t)B * ((n + 7) / 8) * p.tiles_j;
+  if (tiles > 0x7fffffffLL) return fail(MF_ERR_SHAPE, "too many pair tiles");
+  p.tiles = (int)tiles;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  p.per_group = (int)((tiles + cus - 1) / cus);
+  const int groups = (int)((tiles + p.per_group - 1) / p.per_group);
+  p.a = a; p.b = b; p.w = w; p.bias = bias; p.out = out;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kern) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(512), LDS_BYTES, s, p);
+    return hipGetLastError();
+  };
+  return (int)(dtype == MF_DTYPE_BF16 ? launch(opm_fused_kernel<bf16_t>) : launch(opm_fused_kernel<f16_t>));
+}

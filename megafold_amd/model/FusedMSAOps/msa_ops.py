@@ -40,7 +40,7 @@ from ..FusedTriangleAttention.triangle_attention import sigmoid_gate_backward
 from ..gate import sigmoid_gate
 from ..linear import linear_no_bias
 
-__all__ = ["MSAPairWeightedAveraging", "OuterProductMean"]
+__all__ = ["MSAPairWeightedAveraging", "OuterProductMean", "PairWeightedAverageFunction", "OuterProductProjectFunction"]
 
 
 def _pwa_args(b, s, n, h, d, dtype, device):
@@ -219,12 +219,67 @@ class OuterProductMean(nn.Module):
         a = (a.float() * fa).to(dtype)             # one rounding: 1 / rows is not a 16-bit number
         if fb is not None:
             b_ = b_ * fb.to(dtype)
-        # outer[(i d), (j e)] = sum_s a[s, i, d] b[s, j, e]: one GEMM per batch element with the contraction axis
-        # contiguous in both operands
+        # operand matrices [(i d), s] with the contraction axis contiguous
         A = a.permute(0, 2, 3, 1).reshape(b, n * dh, s)
         B = b_.permute(0, 2, 3, 1).reshape(b, n * dh, s)
-        outer = torch.bmm(A, B.transpose(1, 2))                                              # [b, (i d), (j e)]
-        outer = _Permute0213.apply(outer.view(b * n, dh, n, dh)).view(b, n, n, dh * dh)          # "b i j (d e)"
-        out = linear_no_bias(outer, self.to_pairwise_repr.weight)
-        bias = self.to_pairwise_repr.bias
-        return out + bias.to(out.dtype) if bias is not None else out
+        lin = self.to_pairwise_repr
+        if (dh == 32 and lin.out_features == 128 and s <= 128 and dtype in (torch.float16, torch.bfloat16) and A.is_cuda):
+            return OuterProductProjectFunction.apply(A, B, lin.weight, lin.bias, n)
+        return _outer_project_reference(A, B, lin.weight, lin.bias, n, dh)
+
+
+def _outer_project_reference(A, B, weight, bias, n, dh):
+    """The two-GEMM form: ``outer[(i d), (j e)] = A B^T`` per batch element, one layout move to ``"b i j (d e)"``
+    and the projection (shapes the fused kernel does not take, and the backward of the fused forward)."""
+    b = A.shape[0]
+    outer = torch.bmm(A, B.transpose(1, 2))                                                  # [b, (i d), (j e)]
+    outer = _Permute0213.apply(outer.view(b * n, dh, n, dh)).view(b, n, n, dh * dh)          # "b i j (d e)"
+    out = linear_no_bias(outer, weight)
+    return out + bias.to(out.dtype) if bias is not None else out
+
+
+class OuterProductProjectFunction(torch.autograd.Function):
+    """``out[b, i, j, :] = W . (sum_s A[b, (i d), s] B[b, (j e), s])_(d e) + bias`` through ``mf_opm_fused_fwd``: the
+    ``[n, n, dh * dh]`` outer product never exists in the forward.  The backward recomputes it and runs the two-GEMM
+    form under autograd (it holds the outer product while it runs)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx, A, B, weight, bias, n):
+        b, rows, s = A.shape
+        dtype = A.dtype
+        with torch.cuda.device(A.device):
+            # zero padded to 128 columns; the weight with its two hidden indices exchanged (column e * 32 + d)
+            Ap = torch.zeros((b, rows, 128), dtype=dtype, device=A.device)
+            Bp = torch.zeros((b, rows, 128), dtype=dtype, device=A.device)
+            Ap[:, :, :s] = A
+            Bp[:, :, :s] = B
+            wp = weight.to(dtype).view(128, 32, 32).transpose(1, 2).contiguous()
+            out = torch.empty((b, n, n, 128), dtype=dtype, device=A.device)
+            _lib.check(_lib.lib().mf_opm_fused_fwd(Ap.data_ptr(), Bp.data_ptr(), wp.data_ptr(),
+                                                   bias.to(dtype).data_ptr() if bias is not None else None,
+                                                   out.data_ptr(), b, n, _lib.dtype_code(dtype),
+                                                   torch.cuda.current_stream(A.device).cuda_stream),
+                       "mf_opm_fused_fwd")
+        ctx.save_for_backward(A, B, weight, bias)
+        ctx.n = n
+        return out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dout):
+        from ..linear import tall_skinny_tn
+        A, B, weight, bias = ctx.saved_tensors
+        b, rows, s = A.shape
+        n, dh = ctx.n, 32
+        dout2 = dout.reshape(b * n * n, 128).to(A.dtype)
+        w = weight.to(A.dtype)
+        # the outer product again (it was never stored), in the projection's row layout
+        outer = _Permute0213._move(torch.bmm(A, B.transpose(1, 2)).view(b * n, dh, n, dh)).view(b * n * n, dh * dh)
+        dW = tall_skinny_tn(dout2.contiguous(), outer)                            # [128, dh * dh]
+        del outer
+        dbias = dout2.sum(0, dtype=torch.float32).to(bias.dtype) if bias is not None else None
+        douter = _Permute0213._move((dout2 @ w).view(b * n, n, dh, dh)).view(b, rows, rows)   # back to [(i d), (j e)]
+        dA = torch.bmm(douter, B)
+        dB = torch.bmm(douter.transpose(1, 2), A)
+        return dA, dB, dW.to(weight.dtype), dbias, None

@@ -149,7 +149,18 @@ def test_outer_product_mean_at_the_msa_module_size():
     want_out, want_dm, want_dp = om.outer_product_mean_forward_backward(msa, params, dout, mask, msa_mask, dtype=torch.float32)
     m = m.cuda()
     mg = msa.cuda().requires_grad_(True)
-    out = m(mg, mask=mask.cuda(), msa_mask=msa_mask.cuda())
+    dmask, dmsa_mask = mask.cuda(), msa_mask.cuda()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    out = m(mg, mask=dmask, msa_mask=dmsa_mask)
+    torch.cuda.synchronize()
+    # the forward never holds the [n, n, dh * dh] outer product (288 MiB here), neither while it runs nor for the
+    # backward: its peak is the output (36 MiB), the projected MSA and the two operand matrices
+    fwd_peak_mib = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+    held_mib = (torch.cuda.memory_allocated() - base) / 2 ** 20
+    print("outer product mean forward: peak %.0f MiB, held for backward %.0f MiB" % (fwd_peak_mib, held_mib), flush=True)
+    assert fwd_peak_mib < 100 and held_mib < 80
     out.backward(dout.cuda())
     close("out", out, want_out, tol_for(dtype))
     assert rel_rms(out, want_out) < 4e-3
