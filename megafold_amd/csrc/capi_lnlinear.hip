@@ -148,10 +148,9 @@ extern "C" int mf_lnlinear_bwd(const mf_lnlinear_args* a) {
   if (e != hipSuccess) return (int)e;
   const void* dY = a->dout;
   if (a->act == MF_ACT_SWIGLU) {
-    // recompute the pre-activation tile by tile and turn dh into dU = [da, dg]; where the shape allows it the same
-    // pass also forms the weight-gradient partials, so that dU is read back only once (by the dx kernel)
+    // recompute the pre-activation tile by tile and turn dh into dU = [da, dg]; where the shape allows it one pass
+    // forms the weight-gradient partials and dU W'^T per column block, and dU never reaches memory
     e = launch_ln_swiglu_bwd_fused(p, stream);
-    if (e == hipSuccess) return (int)launch_ln_bwd_dx(p, p.du, stream);
     if (e != hipErrorNotSupported) return (int)e;
     e = launch_ln_fwd(p, LN_ACT_SWIGLU_BWD, stream);
     if (e != hipSuccess) return (int)e;

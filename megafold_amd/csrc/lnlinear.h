@@ -56,9 +56,9 @@ struct LnParams {
 bool ln_bwd_takes_dx_add(int dtype, int K, int N);
 hipError_t launch_ln_prep(const LnParams& p, bool forward, hipStream_t stream);
 hipError_t launch_ln_fwd(const LnParams& p, int act, hipStream_t stream);
-// SwiGLU backward: dU (to p.du) and the weight / LayerNorm parameter gradients in one pass + reduction;
+// SwiGLU backward, complete (dx and the weight / LayerNorm parameter gradients; p.du is scratch);
 // hipErrorNotSupported when the shape needs the separate kernels (launch_ln_fwd with LN_ACT_SWIGLU_BWD, then
-// launch_ln_bwd_dw on p.du).
+// launch_ln_bwd_dx and launch_ln_bwd_dw on p.du).
 hipError_t launch_ln_swiglu_bwd_fused(const LnParams& p, hipStream_t stream);
 hipError_t launch_ln_bwd_dx(const LnParams& p, const void* dY, hipStream_t stream);
 hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t stream);

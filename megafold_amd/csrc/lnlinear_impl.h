@@ -360,17 +360,13 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_fwd_kern
   if (it > 0) flush_block(rb - G);
 }
 
-static int g_num_cu = 0;
+// Compute units of the current device, asked at every launch: a process may drive devices of different sizes.
 static inline int num_cu() {
-  if (g_num_cu == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      g_num_cu = n;
-    else
-      g_num_cu = 256;
-  }
-  return g_num_cu;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+    return n;
+  return 256;
 }
 
 template <typename T, int KP, int NTW, int ACT, int WN>
@@ -1168,22 +1164,39 @@ template <typename T> hipError_t ln_dw_dispatch(const LnParams& p, const void* d
 
 namespace mf {
 
-// SwiGLU backward, first kernel (dU and the weight-gradient partials in one pass) followed by the reduction;
-// returns hipErrorNotSupported for shapes the fused kernel does not take (the caller then runs the separate kernels).
+// SwiGLU backward in three kernels: the fused pass (weight-gradient partials, and each column block's share of
+// dy = dU W'^T in place of dU itself), the reduction of the partials, and dx from the shares.  Returns
+// hipErrorNotSupported for shapes the fused kernel does not take (the caller then runs the separate kernels).
+// With MF_LN_DU_FORM the fused pass writes dU and the general dx kernel reads it back (kept for comparison).
 template <typename T> hipError_t ln_swiglu_bwd_fused_dispatch(const LnParams& p, hipStream_t stream) {
   if constexpr (sizeof(T) != 2) {
     return hipErrorNotSupported;
   } else {
     if (!swiglu_bwd_fused_ok<T>(p)) return hipErrorNotSupported;
+#ifdef MF_LN_DU_FORM
+    constexpr bool PARTS = false;
+#else
+    constexpr bool PARTS = true;
+#endif
     hipError_t e;
     switch (p.KP) {
-      case 32: e = launch_swiglu_bwd_fused_k<T, 32>(p, stream); break;
-      case 64: e = launch_swiglu_bwd_fused_k<T, 64>(p, stream); break;
-      case 128: e = launch_swiglu_bwd_fused_k<T, 128>(p, stream); break;
+      case 32: e = launch_swiglu_bwd_fused_k<T, 32, PARTS>(p, stream); break;
+      case 64: e = launch_swiglu_bwd_fused_k<T, 64, PARTS>(p, stream); break;
+      case 128: e = launch_swiglu_bwd_fused_k<T, 128, PARTS>(p, stream); break;
       default: return hipErrorNotSupported;
     }
     if (e != hipSuccess) return e;
-    return launch_dw_reduce<T>(p, stream);
+    e = launch_dw_reduce<T>(p, stream);
+    if (e != hipSuccess) return e;
+    if constexpr (PARTS) {
+      switch (p.KP) {
+        case 32: return launch_dx_parts_k<T, 32>(p, stream);
+        case 64: return launch_dx_parts_k<T, 64>(p, stream);
+        default: return launch_dx_parts_k<T, 128>(p, stream);
+      }
+    } else {
+      return ln_dx_dispatch<T>(p, p.du, stream);
+    }
   }
 }
 

@@ -1,31 +1,36 @@
 // LayerNorm -> SwiGLU backward, first kernel: recompute the pre-activation U = LN(x) W', turn the incoming
-// gradient of h into dU = [da, dg] (fused_transition.py:44-47), write dU for the dx kernel AND accumulate the
-// weight-gradient partials G = x_hat^T dU, s = colsum(dU) in the same pass, so that dU is read back from HBM
-// once (by the dx kernel) instead of twice.
+// gradient of h into dU = [da, dg] (fused_transition.py:44-47) and, in the same pass, use dU for everything that
+// needs it, so that dU itself (M x N elements, eight times the size of x) never reaches HBM:
+//   * the weight-gradient partials G = x_hat^T dU and s = colsum(dU);
+//   * each column block's share of dy = dU W'^T, [rows, K] in the element type of x (PARTS form).  The dx kernel
+//     below adds the N / 256 shares and applies the LayerNorm backward.
+// (With PARTS = false the kernel writes dU instead and the general dx kernel reads it back.)
 //
 // A work-group has eight wavefronts on a block of 32 rows and 128 value + 128 gate columns:
 //  * wavefronts 0-3 ("producers") are the forward kernel's column-stationary wavefronts: each keeps its 32 value
 //    and 32 gate columns of W'^T in registers, recomputes U^T for the row block, applies the SwiGLU derivative
 //    and leaves da / dg as two row-major 32 x 32 tiles in LDS;
-//  * wavefronts 4-7 ("consumers") take the tiles one iteration later: consumer w - 4 streams rows 8 (w - 4) .. + 7
-//    of all four producers' tiles to the dU matrix (256 contiguous bytes per 16 lanes) and, through transposing LDS
-//    reads, uses the two tiles of producer w - 4 as the B operand of G[k, n] += x_hat^T[k, m] dU[m, n]
-//    (x_hat: the normalised rows, staged beside the raw ones), and adds those tiles' column sums.
-// One producer and one consumer share a SIMD: the first is bound by the vector ALU (the activation), the second
-// by the matrix pipe and LDS, so the weight-gradient work runs in issue slots the producer leaves empty.
+//  * wavefronts 4-7 ("consumers") take the tiles one iteration later.  Through transposing LDS reads consumer
+//    w - 4 uses the two tiles of producer w - 4 as the B operand of G[k, n] += x_hat^T[k, m] dU[m, n]
+//    (x_hat: the normalised rows, staged beside the raw ones) and adds those tiles' column sums; with plain row
+//    reads of all four producers' tiles it forms dy^T[k, m] = sum_n W'[k, n] dU[m, n] for k tile w - 4, the W'
+//    fragments coming from registers or from a private LDS slot per lane.
+// One producer and one consumer share a SIMD, so that the matrix-pipe and LDS work of the second runs in issue
+// slots the first (bound by the vector ALU: the activation) leaves empty.
 // Row blocks are dealt round-robin to gridDim.x work-groups per column block; work-group (bx, by) writes range bx
 // of the partial sums, which the usual reduce / finalize kernels consume.
 #pragma once
 
 namespace mf {
 
-template <typename T, int KP>
+template <typename T, int KP, bool PARTS>
 __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnParams p) {
   static_assert(sizeof(T) == 2 && KP <= 128 && KP >= 32, "16-bit element types, 32 <= padded K <= 128");
   using L = LnLayout<T, KP>;
   using frag = frag_t<T>;
   constexpr int KS = KP / 16, CPR = KP / 8, KT = KP / 32;
   constexpr int RB = 32;
+  constexpr int WLDS = KP > 64 ? 16 : 8;            // PARTS: W' fragments per consumer kept in LDS
   constexpr int OSTR = 32 + 8;                      // row stride of a 32-column tile (elements)
   constexpr int TILE = 32 * OSTR;                   // one da or dg tile
   constexpr int PSET = 4 * TILE + 32;               // tiles of one producer: [2 buffers][da, dg], then 64 bytes that
@@ -40,6 +45,7 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
   float* bpL = csL + 4 * 2 * 32;
   T* Ot = reinterpret_cast<T*>(bpL + 4 * 2 * 32);                  // [4 producers][2 buffers][da, dg][32][OSTR]
   T* Dh = Ot + 4 * PSET;                                           // [4 producers][32][OSTR] incoming gradient
+  T* Wl = Dh + 4 * TILE;                                           // PARTS: [4 consumers][WLDS][64 lanes][8] W' fragments
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const bool producer = w < 4;
@@ -83,15 +89,18 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
     bpL[i] = ok ? p.bprime[col] : 0.0f;
   }
 
-  // ---- staging of a row block by all 512 threads: raw rows, row statistics, normalised rows ----------------
+  // ---- staging of a row block by all 512 threads: raw rows, the forward's row statistics, normalised rows ------
   static_assert(RB * CPR <= 512, "one staged chunk per thread");
   const bool stager = tid < RB * CPR;
   const int srow = (stager ? tid : 0) / CPR, sdc = tid % CPR;
-  frag xr;
+  frag xr = frag_zero<T>();
+  float xmu = 0.0f, xrs = 0.0f;
   auto fetch = [&](int64_t rb) {
     int64_t m = rb * RB + srow;
     m = m < p.M ? m : p.M - 1;
     xr = ld8<T>(X + m * p.K + (8 * sdc < p.K ? 8 * sdc : 0));
+    xmu = p.mean[m];
+    xrs = p.rstd[m];
   };
   auto stash = [&](int64_t rb, int buf, int hbuf) {
     if (stager) {                                                  // whole wavefronts: CPR divides 64
@@ -99,26 +108,14 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
       const bool live = m < p.M && 8 * sdc < p.K;
       const frag xv = live ? xr : frag_zero<T>();
       st8<T>(Xs + (buf * RB + srow) * L::XSTR + 8 * sdc, xv);
-      float s = 0.0f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s += to_f(xv[e]);
-      s = group_sum<CPR>(s);
-      const float mu = s / (float)p.K;
-      float d = 0.0f;
-      if (8 * sdc < p.K) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { const float c = to_f(xv[e]) - mu; d += c * c; }
-      }
-      d = group_sum<CPR>(d);
-      const float rs = __builtin_amdgcn_rsqf(d / (float)p.K + p.eps);
       if (sdc == 0) {
-        meanL[buf * RB + srow] = mu;
-        rstdL[buf * RB + srow] = rs;
+        meanL[buf * RB + srow] = xmu;
+        rstdL[buf * RB + srow] = xrs;
       }
-      const float rl = live ? rs : 0.0f;                           // rows / columns past the end contribute nothing
+      const float rl = live ? xrs : 0.0f;                          // rows / columns past the end contribute nothing
       float v[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = (to_f(xv[e]) - mu) * rl;
+      for (int e = 0; e < 8; ++e) v[e] = (to_f(xv[e]) - xmu) * rl;
       st8<T>(Xh + (hbuf * RB + srow) * L::XSTR + 8 * sdc, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
     }
   };
@@ -227,23 +224,89 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
     float csum[2] = {0.0f, 0.0f};
 #pragma unroll
     for (int a = 0; a < KT; ++a) { G[a][0] = acc_zero(); G[a][1] = acc_zero(); }
-    auto consume = [&](const T* tiles, const T* xh) {
+    // PARTS: rows k = 32 pw .. + 31 of W' for the work-group's 256 columns, resident as A operands of
+    // dy^T[k, m] = sum_n W'[k, n] dU[m, n].  Lane row x supplies k = 32 pw + 16 ((x >> 2) & 1) + 4 (x >> 3) + (x & 3),
+    // so that the accumulator of lane (m, g) holds the 16 contiguous k = 32 pw + 16 g .. + 15.
+    // The first WREG fragments stay in registers; the others are parked in LDS, one 16-byte slot per lane (the
+    // registers do not hold all sixteen beside the weight-gradient accumulators).
+    constexpr int WREG = 16 - WLDS;
+    frag wgf[PARTS && WREG > 0 ? WREG : 1];
+    T* wl = Wl + (pw * WLDS * 64 + l) * 8;
+    if constexpr (PARTS) {
+      const T* Wgp = reinterpret_cast<const T*>(p.Wg);
+      const int k = 32 * pw + 16 * ((x >> 2) & 1) + 4 * (x >> 3) + (x & 3);
 #pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        frag bf[2];
+      for (int i = 0; i < 16; ++i) {
+        const int pp = i >> 2, b = (i >> 1) & 1, st = i & 1;
+        const int n = b * Nhalf + (blockIdx.y * 4 + pp) * 32 + 16 * st + 8 * g;
+        const frag wv = k < p.K ? ld8<T>(Wgp + (int64_t)k * p.N + n) : frag_zero<T>();
+        if (i < WREG) wgf[i] = wv; else st8<T>(wl + (i - WREG) * 64 * 8, wv);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) once, so that no wait for these loads is placed inside the loop
+    }
+    // One row block: the weight-gradient products of producer pw's two tiles and, with PARTS, the column block's
+    // share of dy = dU W'^T for k tile pw (all four producers' tiles), in the element type of x, to
+    // part[blockIdx.y][m][KP] (32 contiguous bytes per lane); the dx kernel adds the column blocks' shares.
+    // The dy products form one dependent chain and are issued between the independent weight-gradient products.
+    auto consume = [&](int64_t rbx, int fb, const T* xh) {
+      const T* tiles = Op + fb * (2 * TILE);
+      const bool dyw = PARTS && 32 * pw < KP;
+      f32x16 dacc = acc_zero();
+      // Eight steps (st, a): two dy products (tiles of producer a) and two weight-gradient products (k tile a) each.
+      // The LDS operands of a step are requested one step ahead, into the other of two register sets; without
+      // that every product would wait for a full LDS round trip.
+      frag uf[2][2], wv[2][2], xf[2], bf[2][2];
+      auto request = [&](int j) {
+        const int st = j >> 2, a = j & 3, slot = j & 1;
+        if (a == 0) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          bf[b] = TrRead<T>::read(tiles + b * TILE, OSTR, 16 * st, g, l, plain_chunk(l), x);
-          float s = 0.0f;
+          for (int b = 0; b < 2; ++b) bf[st][b] = TrRead<T>::read(tiles + b * TILE, OSTR, 16 * st, g, l, plain_chunk(l), x);
+        }
+        if (a < KT) xf[slot] = TrRead<T>::read(xh, L::XSTR, 16 * st, g, l, 32 * a + plain_chunk(l), 32 * a + x);
+        if constexpr (PARTS) {
+          if (dyw) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) s += to_f(bf[b][e]);
-          csum[b] += s;
+            for (int b = 0; b < 2; ++b) {
+              const int i = (a * 2 + b) * 2 + st;
+              uf[slot][b] = ld8<T>(Ot + a * PSET + fb * (2 * TILE) + b * TILE + x * OSTR + 16 * st + 8 * g);
+              if (i >= WREG) wv[slot][b] = ld8<T>(wl + (i - WREG) * 64 * 8);
+            }
+          }
+        }
+      };
+      request(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int st = j >> 2, a = j & 3, slot = j & 1;
+        if (j + 1 < 8) request(j + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (a == 0) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += to_f(bf[st][b][e]);
+            csum[b] += s;
+          }
         }
 #pragma unroll
-        for (int a = 0; a < KT; ++a) {
-          const frag xf = TrRead<T>::read(xh, L::XSTR, 16 * st, g, l, 32 * a + plain_chunk(l), 32 * a + x);
-          G[a][0] = mma(xf, bf[0], G[a][0]);
-          G[a][1] = mma(xf, bf[1], G[a][1]);
+        for (int b = 0; b < 2; ++b) {
+          if constexpr (PARTS) {
+            if (dyw) {
+              const int i = (a * 2 + b) * 2 + st;
+              dacc = mma(i < WREG ? wgf[i < WREG ? i : 0] : wv[slot][b], uf[slot][b], dacc);
+            }
+          }
+          if (a < KT) G[a < KT ? a : 0][b] = mma(xf[slot], bf[st][b], G[a < KT ? a : 0][b]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (PARTS) {
+        const int64_t mm = rbx * RB + x;
+        if (dyw && mm < p.M) {
+          T* dst = reinterpret_cast<T*>(p.du) + ((int64_t)blockIdx.y * p.M + mm) * KP + 32 * pw + 16 * g;
+          st8<T>(dst, cvt8<T>(dacc[0], dacc[1], dacc[2], dacc[3], dacc[4], dacc[5], dacc[6], dacc[7]));
+          st8<T>(dst + 8, cvt8<T>(dacc[8], dacc[9], dacc[10], dacc[11], dacc[12], dacc[13], dacc[14], dacc[15]));
         }
       }
     };
@@ -254,14 +317,14 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
       stash(rb + Gx, buf ^ 1, (it + 1) % 3);
       if (rb + 2 * Gx < nrb) fetch(rb + 2 * Gx);
       if (it > 0) {
-        flush(rb - Gx, buf ^ 1);
-        consume(Op + (buf ^ 1) * (2 * TILE), Xh + ((it - 1) % 3) * RB * L::XSTR);
+        if constexpr (!PARTS) flush(rb - Gx, buf ^ 1);
+        consume(rb - Gx, buf ^ 1, Xh + ((it - 1) % 3) * RB * L::XSTR);
       }
     }
     barrier_keep_vm<63>();
     if (it > 0) {
-      flush(rb - Gx, (it - 1) & 1);
-      consume(Op + ((it - 1) & 1) * (2 * TILE), Xh + ((it - 1) % 3) * RB * L::XSTR);
+      if constexpr (!PARTS) flush(rb - Gx, (it - 1) & 1);
+      consume(rb - Gx, (it - 1) & 1, Xh + ((it - 1) % 3) * RB * L::XSTR);
     }
 
     // ---- partial sums of this work-group: range blockIdx.x --------------------------------------------------
@@ -283,20 +346,74 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
   }
 }
 
+// dx from the column blocks' shares of dy (PARTS form of the kernel above): w = sum of the NPART shares in fp32,
+// then the LayerNorm backward dx = (w - x_hat mean_k(x_hat w) - mean_k(w)) rstd (+ dx_add), one 16-byte chunk of a
+// row per thread, KP / 8 threads per row.  Streams x, the shares and dx once: bound by HBM.
+template <typename T, int KP>
+__global__ void __launch_bounds__(256) ln_bwd_dx_parts_kernel(const LnParams p, int nparts) {
+  using frag = frag_t<T>;
+  constexpr int CPR = KP / 8;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t m = item / CPR;
+  const int dc = (int)(item % CPR);
+  if (m >= p.M) return;                                            // whole rows: CPR divides 64, no partial groups
+  const bool live = 8 * dc < p.K;
+  const T* part = reinterpret_cast<const T*>(p.du) + m * KP + 8 * dc;
+  float wv[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  for (int c = 0; c < nparts; ++c) {
+    const frag pv = ld8<T>(part + (int64_t)c * p.M * KP);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wv[e] += to_f(pv[e]);
+  }
+  const frag xv = live ? ld8<T>(reinterpret_cast<const T*>(p.x) + m * p.K + 8 * dc) : frag_zero<T>();
+  const float mu = p.mean[m], rs = p.rstd[m];
+  float xh[8], s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    xh[e] = live ? (to_f(xv[e]) - mu) * rs : 0.0f;
+    wv[e] = live ? wv[e] : 0.0f;
+    s1 += xh[e] * wv[e];
+    s2 += wv[e];
+  }
+  s1 = group_sum<CPR>(s1);
+  s2 = group_sum<CPR>(s2);
+  const float c1 = s1 / (float)p.K, c2 = s2 / (float)p.K;
+  if (live) {
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (wv[e] - (xh[e] * c1 + c2)) * rs;
+    if (p.dx_add) {                                                // summed in fp32, rounded once below
+      const frag rv = ld8<T>(reinterpret_cast<const T*>(p.dx_add) + m * p.K + 8 * dc);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] += to_f(rv[e]);
+    }
+    st8<T>(reinterpret_cast<T*>(p.dx) + m * p.K + 8 * dc, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
+  }
+}
+
+template <typename T, int KP> static hipError_t launch_dx_parts_k(const LnParams& p, hipStream_t stream) {
+  const int nparts = (p.N / 2) / 128;
+  const int64_t items = p.M * (KP / 8);
+  const int64_t blocks = (items + 255) / 256;
+  if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((ln_bwd_dx_parts_kernel<T, KP>), dim3((unsigned)blocks), dim3(256), 0, stream, p, nparts);
+  return hipGetLastError();
+}
+
 // Shapes the fused kernel takes: 16-bit types, 32 <= padded K <= 128, whole 128-column blocks of the value half.
 template <typename T> static bool swiglu_bwd_fused_ok(const LnParams& p) {
   return sizeof(T) == 2 && p.KP >= 32 && p.KP <= 128 && (p.N / 2) % 128 == 0;
 }
 
-template <typename T, int KP> static hipError_t launch_swiglu_bwd_fused_k(const LnParams& p, hipStream_t stream) {
+template <typename T, int KP, bool PARTS> static hipError_t launch_swiglu_bwd_fused_k(const LnParams& p, hipStream_t stream) {
   using L = LnLayout<T, KP>;
   const int gy = (p.N / 2) / 128;
   const size_t smem = (size_t)5 * 32 * L::XSTR * sizeof(T) + (size_t)4 * 32 * 4 + (size_t)2 * 4 * 2 * 32 * 4 +
-                      (size_t)((4 * 2 * 2 + 4) * 32 * 40 + 4 * 32) * sizeof(T);
+                      (size_t)((4 * 2 * 2 + 4) * 32 * 40 + 4 * 32) * sizeof(T) + (PARTS ? (size_t)4 * (KP > 64 ? 16 : 8) * 64 * 16 : 0);
   const size_t wst = (size_t)128 * L::XSTR * sizeof(T);           // weight staging aliases the tiles
   static_assert(sizeof(T) == 2, "");
   if (wst > (size_t)(4 * 2 * 2 + 4) * 32 * 40 * sizeof(T)) return hipErrorInvalidValue;
-  auto kern = ln_swiglu_bwd_fused_kernel<T, KP>;
+  auto kern = ln_swiglu_bwd_fused_kernel<T, KP, PARTS>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
