@@ -36,7 +36,7 @@ LnPlan make_plan(const mf_lnlinear_args* a, bool backward) {
     pl.off_wg = off; off += align256((uint64_t)a->K * a->N * es);
     pl.off_g = off; off += align256((uint64_t)pl.R * a->K * a->N * 4);
     pl.off_s = off; off += align256((uint64_t)pl.R * a->N * 4);
-    if (swiglu) { pl.off_du = off; off += align256((uint64_t)a->M * a->N * es); }
+    if (swiglu) { pl.off_du = off; off += align256(ln_swiglu_bwd_scratch_elems(a->dtype, a->M, a->K, a->N) * es); }
   }
   pl.total = off;
   return pl;

@@ -36,7 +36,8 @@ struct LnParams {
   const void* dout;    // [M, N] (or [M, N/2] with SwiGLU)
   void* dx;            // [M, K]
   const void* dx_add;  // [M, K] or null: added to dx (residual dx kernel only, see ln_bwd_takes_dx_add)
-  void* du;            // [M, N] gradient of the pre-activation (SwiGLU backward scratch)
+  void* du;            // SwiGLU backward scratch, ln_swiglu_bwd_scratch_elems elements: [N / 256, M, KP] shares of
+                       // dU W'^T (fused pass) or [M, N] gradient of the pre-activation
   void* dW;            // [K, N]   parameter gradients: float, or the element type of x when grads_as_x
   void* db;            // [N] or null
   void* dgamma;        // [K]
@@ -60,6 +61,7 @@ hipError_t launch_ln_fwd(const LnParams& p, int act, hipStream_t stream);
 // hipErrorNotSupported when the shape needs the separate kernels (launch_ln_fwd with LN_ACT_SWIGLU_BWD, then
 // launch_ln_bwd_dx and launch_ln_bwd_dw on p.du).
 hipError_t launch_ln_swiglu_bwd_fused(const LnParams& p, hipStream_t stream);
+uint64_t ln_swiglu_bwd_scratch_elems(int dtype, int64_t M, int K, int N);   // elements of p.du that backward needs
 hipError_t launch_ln_bwd_dx(const LnParams& p, const void* dY, hipStream_t stream);
 hipError_t launch_ln_bwd_dw(const LnParams& p, const void* dY, hipStream_t stream);
 hipError_t launch_swiglu_fwd(const void* x, void* y, int64_t M, int Dh, int dtype, hipStream_t stream);

@@ -38,6 +38,17 @@ hipError_t launch_ln_swiglu_bwd_fused(const LnParams& p, hipStream_t stream) {
   }
 }
 
+// Elements of LnParams::du the SwiGLU backward needs: the column blocks' shares of dU W'^T where the fused pass
+// takes the shape (the condition of swiglu_bwd_fused_ok), all of dU otherwise.
+uint64_t ln_swiglu_bwd_scratch_elems(int dtype, int64_t M, int K, int N) {
+  const int KP = ln_padded_k(K);
+#ifndef MF_LN_DU_FORM
+  if ((dtype == MF_BF16 || dtype == MF_F16) && KP >= 32 && KP <= 128 && (N / 2) % 128 == 0)
+    return (uint64_t)(N / 256) * (uint64_t)M * (uint64_t)KP;
+#endif
+  return (uint64_t)M * (uint64_t)N;
+}
+
 hipError_t launch_ln_bwd_dx(const LnParams& p, const void* dY, hipStream_t stream) {
   switch (p.dtype) {
     case MF_BF16: return ln_dx_dispatch<bf16_t>(p, dY, stream);
