@@ -309,6 +309,15 @@ int mf_pwa_softmax_bwd(const mf_pwa_args* a);
 int mf_opm_fused_fwd(const void* a, const void* b, const void* w, const void* bias, void* out, int32_t B, int32_t n,
                      int32_t dtype, void* stream);
 
+/* Gradient of that projection weight, the outer blocks formed again tile by tile and never stored
+ * (autograd of megafold/model/megafold.py:807-812 with respect to to_pairwise_repr.weight):
+ *   dwt[e*32 + d, c] = sum_{b,i,j} (sum_s a[b, i*32 + d, s] * b[b, j*32 + e, s]) * dout[b, i, j, c]
+ *   a, b as above; dout : [B, n, n, 128] (element type of a); dwt : [1024, 128] float, in the index order of w
+ *   transposed; workspace : mf_opm_dw_workspace_bytes(B, n) bytes, 16-byte aligned.  Fixed summation order. */
+uint64_t mf_opm_dw_workspace_bytes(int32_t B, int32_t n);
+int mf_opm_dw(const void* a, const void* b, const void* dout, float* dwt, void* workspace, uint64_t workspace_bytes,
+              int32_t B, int32_t n, int32_t dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * y[a][c][b][:] = x[a][b][c][:] for contiguous arrays of rows of `row_bytes` bytes (a multiple of 16, at most
  * 256): the layout move between the [(i d), (j e)] result of OuterProductMean's contraction and the

@@ -171,6 +171,169 @@ __global__ void __launch_bounds__(512, 1) opm_fused_kernel(const OpmParams p) {
   }
 }
 
+
+// ================================================================================================
+// Gradient of the projection weight:  dWt[e * 32 + d, c] = sum_{b,i,j} outer[b,i,j,d,e] dOut[b,i,j,c]
+// with the outer blocks recomputed tile by tile as in the forward, never stored.  The accumulators of all
+// 1024 x 128 products would fill a compute unit's register file, so a work-group owns a QUARTER of the products
+// (e in [8 q, 8 q + 8): 256 rows of dWt) and forms only those columns of the outer blocks:
+//   stage 1   wavefront w: the 32 x 32 tile  rows d  x  columns (4 positions j, 8 values e)  of row i0 + w over the
+//             MSA rows; laid into LDS as pair rows of 256 products (e_local * 32 + d)
+//   stage 2   wavefront (kt, ch): dWt_q[64 products, 64 channels] += O^T dOut over the 32 pairs of the tile, both
+//             operands through transposing LDS reads (rows = pairs)
+// A tile's operand rows of b (32 rows of 256 bytes) and its 32 rows of dOut arrive by direct loads, double
+// buffered.  Work-group (q, group) walks over a contiguous run of pair tiles and writes its sums to
+// part[group][q]; opm_dw_reduce_kernel adds the groups in a fixed order.
+constexpr int DW_OSTR = 512 + 32;               // bytes between pair rows of the outer-block buffer
+constexpr int DW_LDS_B = 0;                     // two tiles of 32 operand rows x 256 bytes
+constexpr int DW_LDS_D = 2 * 8192;              // two tiles of 32 dOut rows x 256 bytes
+constexpr int DW_LDS_O = 4 * 8192;
+constexpr int DW_LDS_BYTES = DW_LDS_O + 32 * DW_OSTR;
+
+struct OpmDwParams {
+  int B, n, tiles_j, tiles, per_group, groups;
+  const void* a;      // [B, n * 32, 128]
+  const void* b;      // [B, n * 32, 128]
+  const void* dout;   // [B, n, n, 128]
+  float* part;        // [groups][4][256][128]
+  float* dwt;         // [1024][128]
+};
+
+template <typename T>
+__global__ void __launch_bounds__(512, 1) opm_dw_kernel(const OpmDwParams p) {
+  using frag = frag_t<T>;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t512 = threadIdx.x;
+  const int wv = __builtin_amdgcn_readfirstlane(t512 >> 6);
+  const int l = t512 & 63, x = l & 31, g = l >> 5;
+  const int kt = wv & 3, ch = wv >> 2;
+  const int n = p.n;
+  const int q = blockIdx.x & 3, group = blockIdx.x >> 2;
+  const int t_begin = group * p.per_group;
+  const int t_end = min(p.tiles, t_begin + p.per_group);
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) { acc[a][0] = acc_zero(); acc[a][1] = acc_zero(); }
+
+  const unsigned lds0 = (unsigned)(unsigned long)((__attribute__((address_space(3))) unsigned char*)smem);
+  // one direct load per thread and operand: LDS row r = t512 >> 4 (0..31), 16-byte position pos = t512 & 15 holds
+  // chunk pos ^ (r & 15) of the row.  b: row (j0 + (r >> 3)) * 32 + 8 q + (r & 7); dOut: pair (i0 + (r >> 2), j0 + (r & 3))
+  auto issue = [&](int tile, int buf) {
+    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+    const int r = t512 >> 4, pos = t512 & 15, chunk = (pos ^ (r & 15)) << 4;
+    int j = j0 + (r >> 3);
+    j = j < n ? j : n - 1;
+    const char* bbase = reinterpret_cast<const char*>(p.b) + (int64_t)bb * n * 32 * 256;
+    dma16((unsigned)((j * 32 + 8 * q + (r & 7)) * 256 + chunk), bbase, lds0 + DW_LDS_B + buf * 8192 + wv * 1024);
+    int i = i0 + (r >> 2), jd = j0 + (r & 3);
+    i = i < n ? i : n - 1;
+    jd = jd < n ? jd : n - 1;
+    const char* dbase = reinterpret_cast<const char*>(p.dout) + (int64_t)bb * n * n * 256;
+    dma16((unsigned)((i * n + jd) * 256 + chunk), dbase, lds0 + DW_LDS_D + buf * 8192 + wv * 1024);
+  };
+
+  unsigned char* Ob = smem + DW_LDS_O;
+  frag af[8];
+  int cur_i0 = -1, cur_b = -1;
+  if (t_begin < t_end) issue(t_begin, 0);
+  for (int tile = t_begin; tile < t_end; ++tile) {
+    const int buf = (tile - t_begin) & 1;
+    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+    if (i0 != cur_i0 || bb != cur_b) {             // rows d of position i0 + wv (columns of the block: permuted)
+      int i = i0 + wv;
+      i = i < n ? i : n - 1;
+      const T* arow = reinterpret_cast<const T*>(p.a) + ((int64_t)bb * n * 32 + i * 32 + unperm32(x)) * 128 + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) af[ks] = ld8<T>(arow + 16 * ks);
+      cur_i0 = i0; cur_b = bb;
+    }
+    wait_vm<0>();                                  // this tile's rows have arrived
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();                  // ... for every wavefront; the other slots and the outer-block
+    asm volatile("" ::: "memory");                 // buffer are free (their readers are past the preceding tile)
+    if (tile + 1 < t_end) issue(tile + 1, buf ^ 1);
+    // ---- stage 1
+    {
+      const unsigned char* Bt = smem + DW_LDS_B + buf * 8192;
+      f32x16 o = acc_zero();
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const frag bf = ld8<T>(reinterpret_cast<const T*>(Bt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
+        o = mma(af[ks], bf, o);                    // rows = d (16 g + r in register r), columns = (j, e_local) = lane x
+      }
+      const int jj = x >> 3, el = x & 7;
+      const bool live = i0 + wv < n && j0 + jj < n;  // pairs past the edge contribute nothing
+      unsigned char* orow = Ob + (wv * 4 + jj) * DW_OSTR + (el * 32 + 16 * g) * 2;
+      st8<T>(reinterpret_cast<T*>(orow), live ? acc_half<T>(o, 0) : frag_zero<T>());
+      st8<T>(reinterpret_cast<T*>(orow + 16), live ? acc_half<T>(o, 1) : frag_zero<T>());
+    }
+    barrier_keep_vm<63>();                         // LDS hand-over only: the next tile keeps travelling
+    // ---- stage 2
+    {
+      const unsigned char* Dt = smem + DW_LDS_D + buf * 8192;
+      const int a4 = (l >> 2) & 3;
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        frag of[2], df[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          of[u] = TrRead<T>::read(reinterpret_cast<const T*>(Ob), DW_OSTR / 2, 16 * st, g, l,
+                                  kt * 64 + u * 32 + plain_chunk(l), kt * 64 + u * 32 + x);
+          // dOut rows are swizzled: the two 8-byte runs a lane points at lie in rows r0 and r0 + 4
+          const int col = ch * 64 + u * 32 + plain_chunk(l);                 // element column of the run
+          const int r0 = 16 * st + 8 * g + a4, r1 = r0 + 4;
+          const unsigned char* p0 = Dt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
+          const unsigned char* p1 = Dt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+          typedef short s16x8 __attribute__((ext_vector_type(8)));
+          s16x8 v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+          df[u] = __builtin_bit_cast(frag, v);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int c = 0; c < 2; ++c) acc[a][c] = mma(of[a], df[c], acc[a][c]);   // rows = products, columns = channels
+      }
+    }
+  }
+  // ---- this work-group's sums: register r of lane (x, g) is row 8 (r >> 2) + 4 g + (r & 3), column x of its tile
+  float* dst = p.part + ((int64_t)group * 4 + q) * 256 * 128;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = kt * 64 + a * 32 + 8 * (r >> 2) + 4 * g + (r & 3), col = ch * 64 + c * 32 + x;
+        dst[row * 128 + col] = acc[a][c][r];
+      }
+}
+
+// dwt[q * 256 + row][c] = sum over the groups, in their order
+__global__ void __launch_bounds__(256) opm_dw_reduce_kernel(const OpmDwParams p) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;          // float4 index into [1024][128]
+  if (idx >= 1024 * 128 / 4) return;
+  // eight independent loads at a time (a load-add chain would pay the memory latency once per group), fixed order
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  const float* src = p.part + (int64_t)idx * 4;
+  int gidx = 0;
+  for (; gidx + 8 <= p.groups; gidx += 8) {
+    f32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f32x4*>(src + (int64_t)(gidx + u) * 1024 * 128);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; gidx < p.groups; ++gidx) s += *reinterpret_cast<const f32x4*>(src + (int64_t)gidx * 1024 * 128);
+  *reinterpret_cast<f32x4*>(p.dwt + (int64_t)idx * 4) = s;
+}
+
 }  // namespace
 }  // namespace mf
 
@@ -204,4 +367,51 @@ extern "C" int mf_opm_fused_fwd(const void* a, const void* b, const void* w, con
     return hipGetLastError();
   };
   return (int)(dtype == MF_DTYPE_BF16 ? launch(opm_fused_kernel<bf16_t>) : launch(opm_fused_kernel<f16_t>));
+}
+
+static int opm_dw_groups() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  return cus >= 4 ? cus / 4 : 1;
+}
+
+extern "C" uint64_t mf_opm_dw_workspace_bytes(int32_t B, int32_t n) {
+  if (B <= 0 || n <= 0) return 0;
+  return (uint64_t)opm_dw_groups() * 1024 * 128 * 4;
+}
+
+extern "C" int mf_opm_dw(const void* a, const void* b, const void* dout, float* dwt, void* workspace, uint64_t workspace_bytes,
+                         int32_t B, int32_t n, int32_t dtype, void* stream) {
+  clear_error();
+  if (!a || !b || !dout || !dwt || !workspace) return fail(MF_ERR_NULL, "a, b, dout, dwt or workspace is NULL");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(dout) || !aligned16(dwt) || !aligned16(workspace))
+    return fail(MF_ERR_ALIGN, "operands must be 16-byte aligned");
+  if (B <= 0 || n <= 0) return fail(MF_ERR_SHAPE, "B, n must be positive (got %d, %d)", B, n);
+  if ((int64_t)n * 32 * 256 >= (1LL << 31) || (int64_t)n * n * 256 >= (1LL << 31)) return fail(MF_ERR_SHAPE, "n=%d too large", n);
+  if (dtype != MF_DTYPE_F16 && dtype != MF_DTYPE_BF16) return fail(MF_ERR_DTYPE, "dtype %d unsupported: f16 / bf16", dtype);
+  OpmDwParams p{};
+  p.B = B; p.n = n;
+  p.tiles_j = (n + 3) / 4;
+  const int64_t tiles = (int64_t)B * ((n + 7) / 8) * p.tiles_j;
+  if (tiles > 0x7fffffffLL) return fail(MF_ERR_SHAPE, "too many pair tiles");
+  p.tiles = (int)tiles;
+  const int max_groups = opm_dw_groups();
+  p.per_group = (int)((tiles + max_groups - 1) / max_groups);
+  p.groups = (int)((tiles + p.per_group - 1) / p.per_group);
+  if (workspace_bytes < (uint64_t)p.groups * 1024 * 128 * 4)
+    return fail(MF_ERR_WORKSPACE, "mf_opm_dw needs %llu workspace bytes, got %llu", (unsigned long long)p.groups * 1024 * 128 * 4,
+                (unsigned long long)workspace_bytes);
+  p.a = a; p.b = b; p.dout = dout; p.part = static_cast<float*>(workspace); p.dwt = dwt;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kern) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DW_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.groups * 4)), dim3(512), DW_LDS_BYTES, s, p);
+    return hipGetLastError();
+  };
+  hipError_t e = dtype == MF_DTYPE_BF16 ? launch(opm_dw_kernel<bf16_t>) : launch(opm_dw_kernel<f16_t>);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(opm_dw_reduce_kernel, dim3(1024 * 128 / 4 / 256), dim3(256), 0, s, p);
+  return (int)hipGetLastError();
 }

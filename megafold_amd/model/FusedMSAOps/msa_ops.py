@@ -261,23 +261,30 @@ class OuterProductProjectFunction(torch.autograd.Function):
                                                    out.data_ptr(), b, n, _lib.dtype_code(dtype),
                                                    torch.cuda.current_stream(A.device).cuda_stream),
                        "mf_opm_fused_fwd")
-        ctx.save_for_backward(A, B, weight, bias)
-        ctx.n = n
+        ctx.save_for_backward(Ap, Bp, weight, bias)
+        ctx.n, ctx.s = n, s
         return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dout):
-        from ..linear import tall_skinny_tn
-        A, B, weight, bias = ctx.saved_tensors
-        b, rows, s = A.shape
-        n, dh = ctx.n, 32
-        dout2 = dout.reshape(b * n * n, 128).to(A.dtype)
-        w = weight.to(A.dtype)
-        # the outer product again (it was never stored), in the projection's row layout
-        outer = _Permute0213._move(torch.bmm(A, B.transpose(1, 2)).view(b * n, dh, n, dh)).view(b * n * n, dh * dh)
-        dW = tall_skinny_tn(dout2.contiguous(), outer)                            # [128, dh * dh]
-        del outer
+        Ap, Bp, weight, bias = ctx.saved_tensors
+        b, rows, _ = Ap.shape
+        n, dh, s = ctx.n, 32, ctx.s
+        A, B = Ap[:, :, :s], Bp[:, :, :s]
+        dout2 = dout.reshape(b * n * n, 128).to(Ap.dtype).contiguous()
+        w = weight.to(Ap.dtype)
+        # weight gradient: the outer blocks are formed again tile by tile inside mf_opm_dw, never stored;
+        # the kernel returns [e * 32 + d, channel] in fp32
+        lib = _lib.lib()
+        with torch.cuda.device(Ap.device):
+            nbytes = lib.mf_opm_dw_workspace_bytes(b, n)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=Ap.device)
+            dwt = torch.empty((dh * dh, 128), dtype=torch.float32, device=Ap.device)
+            _lib.check(lib.mf_opm_dw(Ap.data_ptr(), Bp.data_ptr(), dout2.data_ptr(), dwt.data_ptr(), ws.data_ptr(), nbytes,
+                                     b, n, _lib.dtype_code(Ap.dtype), torch.cuda.current_stream(Ap.device).cuda_stream),
+                       "mf_opm_dw")
+        dW = dwt.view(dh, dh, 128).permute(2, 1, 0).reshape(128, dh * dh)          # [channel, d * 32 + e]
         dbias = dout2.sum(0, dtype=torch.float32).to(bias.dtype) if bias is not None else None
         douter = _Permute0213._move((dout2 @ w).view(b * n, n, dh, dh)).view(b, rows, rows)   # back to [(i d), (j e)]
         dA = torch.bmm(douter, B)
