@@ -318,6 +318,17 @@ uint64_t mf_opm_dw_workspace_bytes(int32_t B, int32_t n);
 int mf_opm_dw(const void* a, const void* b, const void* dout, float* dwt, void* workspace, uint64_t workspace_bytes,
               int32_t B, int32_t n, int32_t dtype, void* stream);
 
+/* Gradient of one of the two operands, likewise without the [n, n, dh*dh] tensor (autograd of
+ * megafold/model/megafold.py:795-812 with respect to a or b):
+ *   res[b, o*32 + f, s] = sum_{t,h} (sum_c dout[b, pair(o,t), c] * wt[f*32 + h, c]) * opnd[b, t*32 + h, s]
+ *   transposed = 0: pair(o,t) = (o, t): res = da with opnd = b and wt[d*32 + e, c] = W[c, d*32 + e];
+ *   transposed = 1: pair(o,t) = (t, o): res = db with opnd = a and wt[e*32 + d, c] = W[c, d*32 + e].
+ *   dout : [B, n, n, 128]; wt : [1024, 128]; opnd, res : [B, n*32, 128] (all the element type `dtype`, 16 bits);
+ *   workspace : mf_opm_dab_workspace_bytes(B, n) bytes, 16-byte aligned.  Fixed summation order. */
+uint64_t mf_opm_dab_workspace_bytes(int32_t B, int32_t n);
+int mf_opm_dab(const void* dout, const void* wt, const void* opnd, void* res, void* workspace, uint64_t workspace_bytes,
+               int32_t B, int32_t n, int32_t transposed, int32_t dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * y[a][c][b][:] = x[a][b][c][:] for contiguous arrays of rows of `row_bytes` bytes (a multiple of 16, at most
  * 256): the layout move between the [(i d), (j e)] result of OuterProductMean's contraction and the

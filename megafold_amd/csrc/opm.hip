@@ -334,6 +334,189 @@ __global__ void __launch_bounds__(256) opm_dw_reduce_kernel(const OpmDwParams p)
   *reinterpret_cast<f32x4*>(p.dwt + (int64_t)idx * 4) = s;
 }
 
+
+// ================================================================================================
+// Gradients of the two operands.  With o the position on the side of the result (i for da, j for db), t the
+// other position, f / h the hidden indices that go with them:
+//     dO[o,t,f,h]    = sum_c dOut[pair(o,t), c] wt[f * 32 + h, c]          the gradient of the outer block
+//     res[(o f), s]  = sum_{t,h} dO[o,t,f,h] opnd[(t h), s]
+// again without the [n, n, dh * dh] tensor: a tile of dO lives in LDS between two matrix products.
+//   unit        = (batch, block of 8 positions o, half of the 32 values f); its 128 x 128 result stays in registers
+//   job         = a unit and a tile of 4 positions t; a work-group walks over a contiguous run of jobs and writes one
+//                 partial piece per unit it touches (at most two); opm_dab_reduce_kernel adds the pieces of a unit
+//   stage A     wavefront w: dO rows (f_local = 2 w, 2 w + 1) x 32 h for the 32 pairs of the tile, wt resident in
+//               registers (A operand), dOut rows from LDS; laid into LDS as pair rows of 512 values
+//   stage B     wavefront (rt, sh): rows (2 positions o, 16 f) x 64 values s, contraction over (t, h) = 128:
+//               dO rows as plain fragments, the operand rows through transposing LDS reads
+// The tile's 128 operand rows and 32 dOut rows arrive by direct loads, double buffered.
+constexpr int DAB_OSTR = 1024 + 16;             // bytes between pair rows of the dO tile
+constexpr int DAB_LDS_P = 0;                    // two tiles of 128 operand rows x 256 bytes
+constexpr int DAB_LDS_D = 2 * 32768;            // two tiles of 32 dOut rows x 256 bytes
+constexpr int DAB_LDS_O = DAB_LDS_D + 2 * 8192;
+constexpr int DAB_LDS_BYTES = DAB_LDS_O + 32 * DAB_OSTR;
+
+struct OpmDabParams {
+  int B, n, tiles_t, units_per_batch, jobs, per_group, groups, transposed;
+  const void* dout;   // [B, n, n, 128]
+  const void* wt;     // [1024][128], row f * 32 + h
+  const void* opnd;   // [B, n * 32, 128]
+  float* part;        // [groups][2][128][128]
+  void* res;          // [B, n * 32, 128]
+};
+
+template <typename T>
+__global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
+  using frag = frag_t<T>;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t512 = threadIdx.x;
+  const int wv = __builtin_amdgcn_readfirstlane(t512 >> 6);
+  const int l = t512 & 63, x = l & 31, g = l >> 5;
+  const int rt = wv & 3, sh = wv >> 2;
+  const int n = p.n;
+  const int j_begin = blockIdx.x * p.per_group;
+  const int j_end = min(p.jobs, j_begin + p.per_group);
+  if (j_begin >= j_end) return;
+
+  const unsigned lds0 = (unsigned)(unsigned long)((__attribute__((address_space(3))) unsigned char*)smem);
+  auto decode = [&](int job, int& bb, int& o0, int& fh, int& t0) {
+    const int unit = job / p.tiles_t;
+    t0 = (job % p.tiles_t) * 4;
+    bb = unit / p.units_per_batch;
+    const int u = unit % p.units_per_batch;
+    o0 = (u >> 1) * 8;
+    fh = u & 1;
+  };
+  // direct loads of a job's tiles: LDS row r, 16-byte position pos holds chunk pos ^ (r & 15) of the row
+  auto issue = [&](int job, int buf) {
+    int bb, o0, fh, t0;
+    decode(job, bb, o0, fh, t0);
+    const char* pbase = reinterpret_cast<const char*>(p.opnd) + (int64_t)bb * n * 32 * 256;
+#pragma unroll
+    for (int rd = 0; rd < 4; ++rd) {
+      const int q = rd * 512 + t512, row = q >> 4, pos = q & 15;
+      int grow = t0 * 32 + row;
+      grow = grow < n * 32 ? grow : n * 32 - 1;
+      dma16((unsigned)(grow * 256 + ((pos ^ (row & 15)) << 4)), pbase, lds0 + DAB_LDS_P + buf * 32768 + rd * 8192 + wv * 1024);
+    }
+    const int r = t512 >> 4, pos = t512 & 15;
+    int o = o0 + (r >> 2), t = t0 + (r & 3);
+    o = o < n ? o : n - 1;
+    t = t < n ? t : n - 1;
+    const char* dbase = reinterpret_cast<const char*>(p.dout) + (int64_t)bb * n * n * 256;
+    const int pair = p.transposed ? t * n + o : o * n + t;
+    dma16((unsigned)(pair * 256 + ((pos ^ (r & 15)) << 4)), dbase, lds0 + DAB_LDS_D + buf * 8192 + wv * 1024);
+  };
+
+  unsigned char* Ob = smem + DAB_LDS_O;
+  frag wf[2][8];
+  f32x16 acc[2] = {acc_zero(), acc_zero()};
+  int cur_unit = -1, cur_fh = -1, piece = 0;
+  auto flush = [&](int pc) {                       // register r of lane (x, g): row 8 (r >> 2) + 4 g + (r & 3), column x
+    float* dst = p.part + ((int64_t)blockIdx.x * 2 + pc) * 128 * 128;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        dst[(rt * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + sh * 64 + c * 32 + x] = acc[c][r];
+  };
+
+  issue(j_begin, 0);
+  for (int job = j_begin; job < j_end; ++job) {
+    const int buf = (job - j_begin) & 1;
+    int bb, o0, fh, t0;
+    decode(job, bb, o0, fh, t0);
+    const int unit = job / p.tiles_t;
+    if (unit != cur_unit) {
+      if (cur_unit >= 0) {
+        flush(piece);
+        ++piece;
+        acc[0] = acc_zero(); acc[1] = acc_zero();
+      }
+      cur_unit = unit;
+      if (fh != cur_fh) {                          // rows f * 32 + h of wt, h permuted so that a register holds 16 g + r
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const T* wrow = reinterpret_cast<const T*>(p.wt) + (int64_t)((fh * 16 + 2 * wv + a) * 32 + unperm32(x)) * 128 + 8 * g;
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks) wf[a][ks] = ld8<T>(wrow + 16 * ks);
+        }
+        cur_fh = fh;
+      }
+    }
+    wait_vm<0>();                                  // this job's rows (and wt) have arrived
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (job + 1 < j_end) issue(job + 1, buf ^ 1);
+    // ---- stage A
+    {
+      const unsigned char* Dt = smem + DAB_LDS_D + buf * 8192;
+      f32x16 o[2] = {acc_zero(), acc_zero()};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const frag df = ld8<T>(reinterpret_cast<const T*>(Dt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
+        o[0] = mma(wf[0][ks], df, o[0]);           // rows = h (16 g + r in register r), columns = pairs
+        o[1] = mma(wf[1][ks], df, o[1]);
+      }
+      const bool live = t0 + (x & 3) < n;          // pairs past the edge contribute nothing
+      unsigned char* orow = Ob + x * DAB_OSTR;
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int q = 4 * (2 * wv + a) + 2 * g + u;          // 16-byte chunk (f_local * 32 + 16 g + 8 u) / 8
+          st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), live ? acc_half<T>(o[a], u) : frag_zero<T>());
+        }
+    }
+    barrier_keep_vm<63>();                         // LDS hand-over only: the next job's rows keep travelling
+    // ---- stage B
+    {
+      const unsigned char* Pt = smem + DAB_LDS_P + buf * 32768;
+      const int a4 = (l >> 2) & 3;
+      const int ol = 2 * rt + (x >> 4), fl = x & 15;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int q = 4 * fl + 2 * (ks & 1) + g;
+        const frag of = ld8<T>(reinterpret_cast<const T*>(Ob + (ol * 4 + (ks >> 1)) * DAB_OSTR + ((q ^ ((q >> 4) & 3)) << 4)));
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const int col = sh * 64 + c * 32 + plain_chunk(l);
+          const int r0 = 16 * ks + 8 * g + a4, r1 = r0 + 4;
+          const unsigned char* p0 = Pt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
+          const unsigned char* p1 = Pt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+          typedef short s16x8 __attribute__((ext_vector_type(8)));
+          s16x8 v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+          acc[c] = mma(of, __builtin_bit_cast(frag, v), acc[c]);   // rows = (o, f), columns = s
+        }
+      }
+    }
+  }
+  flush(piece);
+}
+
+// res[b][(o0 + R >> 4) * 32 + fh * 16 + (R & 15)][s] = sum of the unit's pieces, in the order of the work-groups
+template <typename T>
+__global__ void __launch_bounds__(256) opm_dab_reduce_kernel(const OpmDabParams p) {
+  const int unit = blockIdx.x >> 4;
+  const int idx = (blockIdx.x & 15) * 256 + threadIdx.x;      // float4 index into [128][128]
+  const int R = idx >> 5, s4 = (idx & 31) * 4;
+  const int bb = unit / p.units_per_batch, u = unit % p.units_per_batch;
+  const int o = (u >> 1) * 8 + (R >> 4), f = (u & 1) * 16 + (R & 15);
+  if (o >= p.n) return;
+  const int jb = unit * p.tiles_t, je = jb + p.tiles_t - 1;
+  f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k = jb / p.per_group; k <= je / p.per_group; ++k) {
+    const int pc = (k * p.per_group) / p.tiles_t == unit ? 0 : 1;   // piece 0 belongs to the unit of the group's first job
+    sum += *reinterpret_cast<const f32x4*>(p.part + (((int64_t)k * 2 + pc) * 128 + R) * 128 + s4);
+  }
+  T* dst = reinterpret_cast<T*>(p.res) + (((int64_t)bb * p.n + o) * 32 + f) * 128 + s4;
+  dst[0] = (T)sum[0]; dst[1] = (T)sum[1]; dst[2] = (T)sum[2]; dst[3] = (T)sum[3];
+}
+
 }  // namespace
 }  // namespace mf
 
@@ -414,4 +597,57 @@ extern "C" int mf_opm_dw(const void* a, const void* b, const void* dout, float* 
   if (e != hipSuccess) return (int)e;
   hipLaunchKernelGGL(opm_dw_reduce_kernel, dim3(1024 * 128 / 4 / 256), dim3(256), 0, s, p);
   return (int)hipGetLastError();
+}
+
+static void opm_dab_plan(OpmDabParams& p, int B, int n) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  p.B = B; p.n = n;
+  p.tiles_t = (n + 3) / 4;
+  p.units_per_batch = ((n + 7) / 8) * 2;
+  const int64_t jobs = (int64_t)B * p.units_per_batch * p.tiles_t;
+  p.jobs = (int)jobs;
+  int per = (int)((jobs + cus - 1) / cus);
+  if (per > p.tiles_t) per = p.tiles_t;            // a work-group then touches at most two units
+  p.per_group = per;
+  p.groups = (int)((jobs + per - 1) / per);
+}
+
+extern "C" uint64_t mf_opm_dab_workspace_bytes(int32_t B, int32_t n) {
+  if (B <= 0 || n <= 0 || (int64_t)B * (((int64_t)n + 7) / 8) * 2 * (((int64_t)n + 3) / 4) > 0x7fffffffLL) return 0;
+  OpmDabParams p{};
+  opm_dab_plan(p, B, n);
+  return (uint64_t)p.groups * 2 * 128 * 128 * 4;
+}
+
+extern "C" int mf_opm_dab(const void* dout, const void* wt, const void* opnd, void* res, void* workspace, uint64_t workspace_bytes,
+                          int32_t B, int32_t n, int32_t transposed, int32_t dtype, void* stream) {
+  clear_error();
+  if (!dout || !wt || !opnd || !res || !workspace) return fail(MF_ERR_NULL, "dout, wt, opnd, res or workspace is NULL");
+  if (!aligned16(dout) || !aligned16(wt) || !aligned16(opnd) || !aligned16(res) || !aligned16(workspace))
+    return fail(MF_ERR_ALIGN, "operands must be 16-byte aligned");
+  if (B <= 0 || n <= 0) return fail(MF_ERR_SHAPE, "B, n must be positive (got %d, %d)", B, n);
+  if ((int64_t)n * 32 * 256 >= (1LL << 31) || (int64_t)n * n * 256 >= (1LL << 31)) return fail(MF_ERR_SHAPE, "n=%d too large", n);
+  if ((int64_t)B * (((int64_t)n + 7) / 8) * 2 * (((int64_t)n + 3) / 4) > 0x7fffffffLL) return fail(MF_ERR_SHAPE, "too many jobs");
+  if (dtype != MF_DTYPE_F16 && dtype != MF_DTYPE_BF16) return fail(MF_ERR_DTYPE, "dtype %d unsupported: f16 / bf16", dtype);
+  OpmDabParams p{};
+  opm_dab_plan(p, B, n);
+  const uint64_t need = (uint64_t)p.groups * 2 * 128 * 128 * 4;
+  if (workspace_bytes < need)
+    return fail(MF_ERR_WORKSPACE, "mf_opm_dab needs %llu workspace bytes, got %llu", (unsigned long long)need, (unsigned long long)workspace_bytes);
+  p.transposed = transposed ? 1 : 0;
+  p.dout = dout; p.wt = wt; p.opnd = opnd; p.part = static_cast<float*>(workspace); p.res = res;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kern, auto red) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, DAB_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.groups), dim3(512), DAB_LDS_BYTES, s, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(red, dim3((unsigned)(B * p.units_per_batch * 16)), dim3(256), 0, s, p);
+    return hipGetLastError();
+  };
+  return (int)(dtype == MF_DTYPE_BF16 ? launch(opm_dab_kernel<bf16_t>, opm_dab_reduce_kernel<bf16_t>)
+                                      : launch(opm_dab_kernel<f16_t>, opm_dab_reduce_kernel<f16_t>));
 }

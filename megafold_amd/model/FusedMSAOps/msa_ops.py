@@ -286,7 +286,17 @@ class OuterProductProjectFunction(torch.autograd.Function):
                        "mf_opm_dw")
         dW = dwt.view(dh, dh, 128).permute(2, 1, 0).reshape(128, dh * dh)          # [channel, d * 32 + e]
         dbias = dout2.sum(0, dtype=torch.float32).to(bias.dtype) if bias is not None else None
-        douter = _Permute0213._move((dout2 @ w).view(b * n, n, dh, dh)).view(b, rows, rows)   # back to [(i d), (j e)]
-        dA = torch.bmm(douter, B)
-        dB = torch.bmm(douter.transpose(1, 2), A)
+        # operand gradients: tiles of dOut . W^T live in LDS between two products inside mf_opm_dab (once per side)
+        with torch.cuda.device(Ap.device):
+            wt_a = w.t().contiguous()                                                        # row d * 32 + e
+            wt_b = w.view(128, dh, dh).permute(2, 1, 0).reshape(dh * dh, 128).contiguous()   # row e * 32 + d
+            nbytes = lib.mf_opm_dab_workspace_bytes(b, n)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=Ap.device)
+            dAp, dBp = torch.empty_like(Ap), torch.empty_like(Bp)
+            stream = torch.cuda.current_stream(Ap.device).cuda_stream
+            _lib.check(lib.mf_opm_dab(dout2.data_ptr(), wt_a.data_ptr(), Bp.data_ptr(), dAp.data_ptr(), ws.data_ptr(), nbytes,
+                                      b, n, 0, _lib.dtype_code(Ap.dtype), stream), "mf_opm_dab")
+            _lib.check(lib.mf_opm_dab(dout2.data_ptr(), wt_b.data_ptr(), Ap.data_ptr(), dBp.data_ptr(), ws.data_ptr(), nbytes,
+                                      b, n, 1, _lib.dtype_code(Ap.dtype), stream), "mf_opm_dab")
+        dA, dB = dAp[:, :, :s], dBp[:, :, :s]
         return dA, dB, dW.to(weight.dtype), dbias, None
