@@ -10,18 +10,19 @@ parameter names::
     OuterProductMean           to_hidden.{WEIGHT,BIAS,linear_weight}                   LayernormLinear(dim_msa, 2*dim_hidden)
                                to_pairwise_repr.weight / .bias                         Linear(dim_hidden^2, dim_pairwise)
 
-``MSAPairWeightedAveraging``: ``out[b,s,i,h,:] = sum_j softmax_j(bias[b,h,i,j] + mask[j]) values[b,s,j,h,:]`` is
-the pair-biased attention operator with zero queries and keys and the MSA rows as its row batch: the pair
-bias is shared by every row, which is exactly what the attention kernels are organised around (one bias tile
-serves several rows).  Values are the strided view of the fused projection output (no ``"b s n (gv h d) ->
-gv b h s n d"`` copy), the result comes out as ``"b s n (h d)"`` (no merge copy), the gate is read in place.
-The wasted Q K^T products (queries and keys are zero) are the price of reusing the tested kernels, including
-their backward (dV and the bias gradient are exactly what this operator needs).
+``MSAPairWeightedAveraging``: ``out[b,s,i,h,:] = sum_j softmax_j(bias[b,h,i,j] + mask[j]) values[b,s,j,h,:]``.  The
+weights do not depend on the MSA row: for the module's shape (16-bit, 8 heads of 32 channels, n <= 384) the softmax is
+taken once per (b, h, i) and the averaging, the gate and the backward run in kernels of their own (``mf_pwa_*``,
+``PairWeightedAverageFunction``).  Other shapes use the pair-biased attention operator with zero queries and keys
+and the MSA rows as its row batch.  Values and gates are column halves of the fused projection output (no
+``"b s n (gv h d) -> gv b h s n d"`` copy), the result comes out as ``"b s n (h d)"`` (no merge copy).
 
-``OuterProductMean``: the fused LayerNorm -> Linear, then the ``s``-contraction as one GEMM of ``[n*dh, s] x
-[s, n*dh]`` per batch element, one layout move to ``"b i j (d e)"`` and the output projection.  The masks and the
-division by the number of MSA rows are folded into the two small operands (exact for the 0/1 masks; the division
-is then rounded before the product instead of after it).
+``OuterProductMean``: the fused LayerNorm -> Linear, the masks and the division by the number of MSA rows folded into
+the two small operands (exact for the 0/1 masks; the division is rounded once, before the product), then for the
+module's shape (16-bit, hidden 32, 128 pair channels) the contraction over the MSA rows and the output projection in
+one kernel (``mf_opm_fused_fwd``) and the backward in three (``mf_opm_dw``, ``mf_opm_dab`` once per operand): the
+``[n, n, hidden^2]`` outer product is never written to memory.  Other shapes run the reference's expressions (one
+GEMM per batch element, a layout move to ``"b i j (d e)"``, the projection).
 """
 from __future__ import annotations
 
@@ -240,8 +241,8 @@ def _outer_project_reference(A, B, weight, bias, n, dh):
 
 class OuterProductProjectFunction(torch.autograd.Function):
     """``out[b, i, j, :] = W . (sum_s A[b, (i d), s] B[b, (j e), s])_(d e) + bias`` through ``mf_opm_fused_fwd``: the
-    ``[n, n, dh * dh]`` outer product never exists in the forward.  The backward recomputes it and runs the two-GEMM
-    form under autograd (it holds the outer product while it runs)."""
+    ``[n, n, dh * dh]`` outer product never exists, in the forward or in the backward (``mf_opm_dw`` for the weight,
+    ``mf_opm_dab`` for each operand: the outer blocks and their gradient are formed tile by tile in LDS)."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)

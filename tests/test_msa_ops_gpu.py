@@ -161,7 +161,17 @@ def test_outer_product_mean_at_the_msa_module_size():
     held_mib = (torch.cuda.memory_allocated() - base) / 2 ** 20
     print("outer product mean forward: peak %.0f MiB, held for backward %.0f MiB" % (fwd_peak_mib, held_mib), flush=True)
     assert fwd_peak_mib < 100 and held_mib < 80
-    out.backward(dout.cuda())
+    dd = dout.cuda()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base_b = torch.cuda.memory_allocated()
+    out.backward(dd)
+    torch.cuda.synchronize()
+    # nor does the backward: its three kernels form the outer blocks and their gradient tile by tile (the two-GEMM form
+    # held two 288 MiB tensors at its peak)
+    bwd_peak_mib = (torch.cuda.max_memory_allocated() - base_b) / 2 ** 20
+    print("outer product mean backward: peak %.0f MiB above what the forward left" % bwd_peak_mib, flush=True)
+    assert bwd_peak_mib < 120
     close("out", out, want_out, tol_for(dtype))
     assert rel_rms(out, want_out) < 4e-3
     close("dmsa", mg.grad, want_dm, param_grad_tol(dtype, n, want_dm))
