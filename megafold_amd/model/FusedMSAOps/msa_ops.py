@@ -231,7 +231,7 @@ class OuterProductMean(nn.Module):
 
 def _outer_project_reference(A, B, weight, bias, n, dh):
     """The two-GEMM form: ``outer[(i d), (j e)] = A B^T`` per batch element, one layout move to ``"b i j (d e)"``
-    and the projection (shapes the fused kernel does not take, and the backward of the fused forward)."""
+    and the projection (shapes the fused kernels do not take)."""
     b = A.shape[0]
     outer = torch.bmm(A, B.transpose(1, 2))                                                  # [b, (i d), (j e)]
     outer = _Permute0213.apply(outer.view(b * n, dh, n, dh)).view(b, n, n, dh * dh)          # "b i j (d e)"

@@ -299,3 +299,63 @@ def test_permute_argument_errors():
     assert lib.mf_permute_0213(0x10008, 0x20000, 4, 32, 48, 64, None) == -5
     assert lib.mf_permute_0213(0x10000, 0x20000, 70000, 32, 48, 64, None) == -2 and "grid" in lib.mf_last_error().decode()
     assert len(ok) == 7
+
+
+def test_outer_product_mean_argument_errors():
+    """mf_opm_fused_fwd / mf_opm_dw / mf_opm_dab reject bad arguments before any launch."""
+    lib = _lib.lib()
+    A, Bm, W, O, D, WS = 0x10000, 0x20000, 0x30000, 0x40000, 0x50000, 0x60000
+    bf16 = _lib.MF_BF16
+    assert lib.mf_opm_fused_fwd(None, Bm, W, None, O, 1, 16, bf16, None) == -1
+    assert lib.mf_opm_fused_fwd(A + 8, Bm, W, None, O, 1, 16, bf16, None) == -5
+    assert lib.mf_opm_fused_fwd(A, Bm, W, None, O, 0, 16, bf16, None) == -2
+    assert lib.mf_opm_fused_fwd(A, Bm, W, None, O, 1, 16, _lib.MF_F32, None) == -3 and "f16 / bf16" in lib.mf_last_error().decode()
+    need = lib.mf_opm_dw_workspace_bytes(1, 16)
+    assert need > 0 and need % (1024 * 128 * 4) == 0 and lib.mf_opm_dw_workspace_bytes(0, 16) == 0
+    assert lib.mf_opm_dw(A, Bm, D, None, WS, need, 1, 16, bf16, None) == -1
+    assert lib.mf_opm_dw(A, Bm, D, O + 4, WS, need, 1, 16, bf16, None) == -5
+    assert lib.mf_opm_dw(A, Bm, D, O, WS, need, 1, 16, _lib.MF_F32, None) == -3
+    assert lib.mf_opm_dw(A, Bm, D, O, WS, need, 1, 40000, bf16, None) == -2 and "too large" in lib.mf_last_error().decode()
+    assert lib.mf_opm_dw(A, Bm, D, O, WS, 1024, 1, 16, bf16, None) == -6 and "workspace bytes" in lib.mf_last_error().decode()
+    need = lib.mf_opm_dab_workspace_bytes(2, 37)
+    assert need > 0 and need % (2 * 128 * 128 * 4) == 0 and lib.mf_opm_dab_workspace_bytes(1, -3) == 0
+    assert lib.mf_opm_dab(D, W, None, O, WS, need, 2, 37, 0, bf16, None) == -1
+    assert lib.mf_opm_dab(D, W, Bm, O, WS + 2, need, 2, 37, 0, bf16, None) == -5
+    assert lib.mf_opm_dab(D, W, Bm, O, WS, need - 1, 2, 37, 1, bf16, None) == -6
+    assert lib.mf_opm_dab(D, W, Bm, O, WS, need, 2, 37, 1, 7, None) == -3
+
+
+def test_pair_weighted_averaging_argument_errors():
+    """The mf_pwa_* entry points reject shapes their kernels do not take, unaligned or missing operands and a chunk
+    count that differs from what mf_pwa_dw_chunks reports."""
+    lib = _lib.lib()
+
+    def args(**kw):
+        a = _lib.PwaArgs()
+        a.B, a.S, a.N, a.H, a.D, a.dtype = 1, 6, 40, 8, 32, _lib.MF_BF16
+        a.logits, a.ld_logits = 0x10000, 8
+        a.w = 0x20000
+        a.x, a.ldx = 0x30000, 512
+        a.y, a.ldy = 0x40000, 256
+        a.dy, a.lddy = 0x50000, 256
+        a.dw_part = 0x60000
+        a.dlogits, a.ld_dlogits = 0x70000, 8
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    assert lib.mf_pwa_softmax_fwd(C.byref(args(H=4))) == -2          # eight heads of 32 channels only
+    assert lib.mf_pwa_softmax_fwd(C.byref(args(dtype=_lib.MF_F32))) == -3
+    assert lib.mf_pwa_softmax_fwd(C.byref(args(logits=None))) == -1
+    assert lib.mf_pwa_softmax_fwd(C.byref(args(ld_logits=12))) == -4
+    assert lib.mf_pwa_apply(C.byref(args(N=400))) == -2 and "at most 384" in lib.mf_last_error().decode()
+    assert lib.mf_pwa_apply(C.byref(args(y=None))) == -1
+    assert lib.mf_pwa_apply(C.byref(args(ldy=100))) == -4
+    a = args()
+    n = lib.mf_pwa_dw_chunks(C.byref(a))
+    assert 1 <= n <= 6
+    a.n_chunks = n + 1
+    assert lib.mf_pwa_dw(C.byref(a)) == -6 and "mf_pwa_dw_chunks" in lib.mf_last_error().decode()
+    assert lib.mf_pwa_dw(C.byref(args(dy=None, n_chunks=n))) == -1
+    assert lib.mf_pwa_softmax_bwd(C.byref(args(n_chunks=0))) == -1
+    assert lib.mf_pwa_softmax_bwd(C.byref(args(n_chunks=n, dlogits=0x70004))) == -1
