@@ -877,6 +877,17 @@ template <typename T> hipError_t ln_dx_dispatch(const LnParams& p, const void* d
 // =================================================================================================
 // backward: G = x_hat^T dOut, s = colsum(dOut), then dW / dgamma / dbeta / db
 // =================================================================================================
+// Row stride (elements) of the dW kernel's LDS tiles.  The tiles are read with transposing reads: a group of 16
+// lanes touches 32 contiguous bytes in each of four consecutive rows, so the rows must start 8 banks (32 bytes modulo
+// 256) apart or further; a stride of 4 banks (widths that are multiples of 128 16-bit elements, padded by one
+// 16-byte unit) made every such read a two-way bank conflict.
+template <typename T> constexpr int dw_tile_stride(int width) {
+  constexpr int UNIT = 16 / (int)sizeof(T);
+  int stride = ((width / UNIT) % 2 == 0) ? width + UNIT : width;
+  if (sizeof(T) == 2 && (stride * (int)sizeof(T) / 4) % 64 == 4) stride += UNIT;
+  return stride;
+}
+
 template <int KP> struct DwShape {
   static constexpr int KPT = KP < 32 ? 32 : KP;
   static constexpr int WK = KPT >= 256 ? 4 : (KPT >= 64 ? 2 : 1);   // wavefronts along k
@@ -893,8 +904,8 @@ __global__ void __launch_bounds__(256, 2) ln_bwd_dw_kernel(const LnParams p, con
   constexpr int KPT = Sh::KPT, KTW = Sh::KTW, WNN = Sh::WNN, NTW = Sh::NTW, CW = Sh::CW;
   constexpr int RT = 64;                       // rows per staged tile
   constexpr int UNIT = 16 / (int)sizeof(T);
-  constexpr int XSTR = ((KPT / UNIT) % 2 == 0) ? KPT + UNIT : KPT;
-  constexpr int YSTR = ((CW / UNIT) % 2 == 0) ? CW + UNIT : CW;
+  constexpr int XSTR = dw_tile_stride<T>(KPT);
+  constexpr int YSTR = dw_tile_stride<T>(CW);
   constexpr int XI = RT * (KPT / 8), YI = RT * (CW / 8);
   constexpr int PFX = (XI + 255) / 256, PFY = (YI + 255) / 256;
   static_assert(256 % (CW / 8) == 0, "a thread must keep one column chunk");
@@ -1117,8 +1128,8 @@ template <typename T> static hipError_t launch_dw_reduce(const LnParams& p, hipS
 template <typename T, int KP> static hipError_t launch_dw_t(const LnParams& p, const void* dY, hipStream_t stream) {
   using Sh = DwShape<KP>;
   constexpr int UNIT = 16 / (int)sizeof(T);
-  constexpr int XSTR = ((Sh::KPT / UNIT) % 2 == 0) ? Sh::KPT + UNIT : Sh::KPT;
-  constexpr int YSTR = ((Sh::CW / UNIT) % 2 == 0) ? Sh::CW + UNIT : Sh::CW;
+  constexpr int XSTR = dw_tile_stride<T>(Sh::KPT);
+  constexpr int YSTR = dw_tile_stride<T>(Sh::CW);
   size_t smem = (size_t)2 * 64 * (XSTR + YSTR) * sizeof(T);
   if (smem < 256 * 8 * 4) smem = 256 * 8 * 4;
   const int gy = (p.N + Sh::CW - 1) / Sh::CW;
