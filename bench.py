@@ -394,7 +394,8 @@ def main():
     # by events on the launch stream: every event costs a few microseconds of stream time, and eight of
     # them per step (all four phases) would add 8 % to the step.  The per-phase breakdown is taken in a
     # second, untimed loop below.
-    names = ("fwd", "prep", "dqkv", "dbias")   # "prep" = the backward call's own copy of the pair bias
+    # "prep" = the backward call's own copy of the pair bias: no launch when the forward left its tiles (as here)
+    names = ("fwd", "prep", "dqkv", "dbias")
     DOMINANT = "dqkv"
 
     def step(marks, phases):
@@ -402,7 +403,9 @@ def main():
         if "fwd" in phases:
             ev["fwd"] = [torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)]
             ev["fwd"][0].record()
-        O, lse, (Q, K_, V, mask, bias_) = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"])
+        # as the autograd operator does: the forward leaves the pair bias in the backward's tile order as well
+        O, lse, (Q, K_, V, mask, bias_, tiles) = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"],
+                                                                      save_bias_tiles=True)
         if "fwd" in phases:
             ev["fwd"][1].record()
 
@@ -412,7 +415,7 @@ def main():
                 e.record()
                 ev.setdefault(name, []).append(e)
 
-        evoattention_backward(dev["dO"], Q, K_, V, mask, bias_, O, lse, True, phase_hook=hook)
+        evoattention_backward(dev["dO"], Q, K_, V, mask, bias_, O, lse, True, phase_hook=hook, bias_tiles=tiles)
         if marks is not None:
             marks.append(ev)
 

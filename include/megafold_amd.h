@@ -103,10 +103,17 @@ typedef struct mf_evoattn_args {
   void* workspace;
   uint64_t workspace_bytes;
   void* stream;
+  /* optional, NULL = unused: mf_evoattn_bias_tiles_bytes() bytes, 16-byte aligned.  The forward then also leaves
+   * the pair bias in the tiled fp32 order the backward reads (one launch prepares both orders); a backward
+   * call given the same buffer reads it instead of preparing its own copy, needs a smaller workspace and no
+   * MF_EVO_BWD_PREP phase.  The buffer is an activation the caller keeps between the two calls (the reference
+   * keeps the bias itself, evoattention.py:777); scale, shape and bias must be those of the forward call. */
+  void* bias_tiles_bwd;
 } mf_evoattn_args;
 
 uint64_t mf_evoattn_fwd_workspace_bytes(const mf_evoattn_args* a);
 uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a);
+uint64_t mf_evoattn_bias_tiles_bytes(const mf_evoattn_args* a);
 int mf_evoattn_fwd(const mf_evoattn_args* a);
 int mf_evoattn_bwd(const mf_evoattn_args* a);
 

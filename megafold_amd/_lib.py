@@ -34,6 +34,7 @@ class EvoAttnArgs(C.Structure):
         ("dbias", C.c_void_p),
         ("do_stride", I64x4), ("dq_stride", I64x4), ("dk_stride", I64x4), ("dv_stride", I64x4),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("stream", C.c_void_p),
+        ("bias_tiles_bwd", C.c_void_p),
     ]
 
 
@@ -86,6 +87,7 @@ SYMBOLS = {
     "mf_last_error": (C.c_char_p, []),
     "mf_evoattn_fwd_workspace_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_bwd_workspace_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
+    "mf_evoattn_bias_tiles_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_fwd": (C.c_int, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_bwd": (C.c_int, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_fwd_noalloc": (C.c_int, [C.POINTER(EvoAttnArgs)]),

@@ -24,7 +24,8 @@ Plan make_plan(const mf_evoattn_args* a, bool backward) {
   pl.bias_nt = (a->S + 31) / 32;
   uint64_t off = 0;
   pl.off_bias = off;
-  off += align256((uint64_t)a->B * a->H * pl.bias_nt * pl.bias_nt * 4096);
+  // the backward reads the tiles a forward call left in bias_tiles_bwd, if the caller kept them
+  if (!(backward && a->bias_tiles_bwd)) off += align256((uint64_t)a->B * a->H * pl.bias_nt * pl.bias_nt * 4096);
   pl.n_chunks = 1;
   pl.rows_per_chunk = a->N;
   if (backward) {
@@ -100,9 +101,13 @@ int fill_params(const mf_evoattn_args* a, const Plan& pl, EvoParams& p, hipStrea
   unsigned char* ws = static_cast<unsigned char*>(a->workspace);
   float* b32 = reinterpret_cast<float*>(ws + pl.off_bias);
   if (a->scale <= 0.0f) return fail(MF_ERR_SHAPE, "scale must be positive (got %g)", (double)a->scale);
-  if (prep) {
+  if (a->bias_tiles_bwd && !aligned16(a->bias_tiles_bwd)) return fail(MF_ERR_ALIGN, "bias_tiles_bwd is not 16-byte aligned");
+  if (backward && a->bias_tiles_bwd) {
+    b32 = static_cast<float*>(a->bias_tiles_bwd);          // prepared by the forward: nothing to do here
+  } else if (prep) {
     hipError_t e = launch_bias_prep(a->bias, a->bias_dtype, a->bias_stride[0], a->bias_stride[1], a->bias_stride[2],
-                                    a->bias_stride[3], b32, a->B, a->H, a->S, 1.0f / a->scale, backward, stream);
+                                    a->bias_stride[3], b32, a->B, a->H, a->S, 1.0f / a->scale, backward, stream,
+                                    backward ? nullptr : static_cast<float*>(a->bias_tiles_bwd));
     if (e != hipSuccess) return (int)e;
   }
   p.bias = b32;
@@ -120,6 +125,11 @@ extern "C" const char* mf_last_error(void) { return last_error_buf(); }
 extern "C" uint64_t mf_evoattn_fwd_workspace_bytes(const mf_evoattn_args* a) {
   if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0) return 0;
   return make_plan(a, false).total;
+}
+extern "C" uint64_t mf_evoattn_bias_tiles_bytes(const mf_evoattn_args* a) {
+  if (!a || a->B <= 0 || a->S <= 0 || a->H <= 0) return 0;
+  const uint64_t nt = ((uint64_t)a->S + 31) / 32;
+  return align256((uint64_t)a->B * a->H * nt * nt * 4096);
 }
 extern "C" uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a) {
   if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0) return 0;

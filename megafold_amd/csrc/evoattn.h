@@ -71,7 +71,8 @@ hipError_t launch_evo_bwd_dqkv_pw(const EvoParams& p, int num_cu, hipStream_t st
 // bias (any float dtype, any strides) * mult -> the tiled fp32 copy described at EvoParams::bias;
 // `backward_layout` selects which of the two orders is written.
 hipError_t launch_bias_prep(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
-                            int B, int H, int S, float mult, bool backward_layout, hipStream_t stream);
+                            int B, int H, int S, float mult, bool backward_layout, hipStream_t stream,
+                            float* dst_bwd = nullptr);   // dst_bwd: the backward's order too, in the same launch
 
 // Number of rows of N one work-group of the bias-gradient kernel walks over, chosen so the grid
 // fills the device while the partial-sum workspace stays small.

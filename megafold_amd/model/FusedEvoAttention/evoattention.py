@@ -97,9 +97,12 @@ def _check_inputs(Q, K, V) -> None:
         raise RuntimeError("EvoformerAttention runs on the GPU only (got device %s)" % Q.device)
 
 
-def evoattention_forward(Q, K, V, res_mask, pair_bias, out=None):
+def evoattention_forward(Q, K, V, res_mask, pair_bias, out=None, save_bias_tiles=False):
     """O, LSE = forward.  Returns also the tensors exactly as the kernels saw them.  ``out``: optional
-    ``[B, N, S, H, D]`` tensor to receive O (any strides the kernels accept, e.g. a transposed view)."""
+    ``[B, N, S, H, D]`` tensor to receive O (any strides the kernels accept, e.g. a transposed view).
+    ``save_bias_tiles``: the forward's bias preparation also writes the tiled copy the backward reads; it is
+    returned as a sixth saved tensor, to be passed to ``evoattention_backward(..., bias_tiles=)``, which then skips
+    its own preparation launch (the copy replaces the same number of bytes in the backward's workspace)."""
     _check_inputs(Q, K, V)
     B, N, S, H, D = Q.shape
     if out is not None and (tuple(out.shape) != (B, N, S, H, D) or out.dtype != Q.dtype or not _strided_ok(out)):
@@ -117,7 +120,13 @@ def evoattention_forward(Q, K, V, res_mask, pair_bias, out=None):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=Q.device) if nbytes else None
         a.workspace = ws.data_ptr() if ws is not None else None
         a.workspace_bytes = nbytes
+        tiles = None
+        if save_bias_tiles:
+            tiles = torch.empty(lib.mf_evoattn_bias_tiles_bytes(C.byref(a)), dtype=torch.uint8, device=Q.device)
+            a.bias_tiles_bwd = tiles.data_ptr()
         _lib.check(lib.mf_evoattn_fwd(C.byref(a)), "mf_evoattn_fwd")
+    if save_bias_tiles:
+        return O, lse, (Q, K, V, mask, bias, tiles)
     return O, lse, (Q, K, V, mask, bias)
 
 
@@ -143,12 +152,13 @@ def evoattention_forward_noalloc(Q, K, V, res_mask, pair_bias, O, lse) -> None:
         _lib.check(_lib.lib().mf_evoattn_fwd_noalloc(C.byref(a)), "mf_evoattn_fwd_noalloc")
 
 
-def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None, out=None):
+def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None, out=None, bias_tiles=None):
     """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state.
 
     ``out = (dQ, dK, dV)``, if given, are the tensors to write (``[B, N, S, H, D]`` in Q's dtype, unit
     stride on D and 16-byte multiples elsewhere, e.g. column slices of a wider matrix); otherwise
-    contiguous tensors are allocated.
+    contiguous tensors are allocated.  ``bias_tiles``: the sixth saved tensor of
+    ``evoattention_forward(..., save_bias_tiles=True)`` for the same inputs.
 
     ``phase_hook(name)``, if given, is called before and after each backward phase ("prep", "dqkv",
     "dbias"), which are then enqueued by separate C-ABI calls (used by the benchmark to bracket each
@@ -177,6 +187,8 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phas
         a.dq_stride = _lib.I64x4(*dQ.stride()[:4])
         a.dk_stride = _lib.I64x4(*dK.stride()[:4])
         a.dv_stride = _lib.I64x4(*dV.stride()[:4])
+        if bias_tiles is not None:
+            a.bias_tiles_bwd = bias_tiles.data_ptr()
         nbytes = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=Q.device)
         a.workspace = ws.data_ptr()
@@ -200,16 +212,16 @@ class EvoformerAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, Q, K, V, res_mask, pair_bias):
-        O, lse, (Qs, Ks, Vs, mask, bias) = evoattention_forward(Q, K, V, res_mask, pair_bias)
-        ctx.save_for_backward(Qs, Ks, Vs, mask, bias, O, lse)
+        O, lse, (Qs, Ks, Vs, mask, bias, tiles) = evoattention_forward(Q, K, V, res_mask, pair_bias, save_bias_tiles=True)
+        ctx.save_for_backward(Qs, Ks, Vs, mask, bias, O, lse, tiles)
         ctx.bias_shape = tuple(pair_bias.shape)
         return O
 
     @staticmethod
     def backward(ctx, dO):
-        Q, K, V, mask, bias, O, lse = ctx.saved_tensors
+        Q, K, V, mask, bias, O, lse, tiles = ctx.saved_tensors
         need_dbias = ctx.needs_input_grad[4]
-        dQ, dK, dV, dbias = evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias)
+        dQ, dK, dV, dbias = evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias, bias_tiles=tiles)
         if dbias is not None:
             if ctx.bias_shape[0] == 1 and dbias.shape[0] != 1:
                 dbias = dbias.sum(0, keepdim=True)

@@ -149,8 +149,9 @@ class TriangleAttentionFunction(torch.autograd.Function):
         else:
             mask5 = mask.to(torch.bool).view(b, 1, 1, 1, n)
         O = torch.empty((b, n, n, heads, dim_head), dtype=dt, device=x.device)      # indexed by pair position
-        _, lse, (Qs, Ks, Vs, masks, biass) = evoattention_forward(Q, K, V, mask5, Bv,
-                                                                  out=O.transpose(1, 2) if transposed else O)
+        _, lse, (Qs, Ks, Vs, masks, biass, tiles) = evoattention_forward(Q, K, V, mask5, Bv,
+                                                                         out=O.transpose(1, 2) if transposed else O,
+                                                                         save_bias_tiles=True)
         O2d = O.view(b * n * n, inner)
         A = sigmoid_gate_forward(O2d, G)
         out = F.linear(A, Wo.to(dt))
@@ -160,7 +161,7 @@ class TriangleAttentionFunction(torch.autograd.Function):
             # the LayerNorm backward below.
             out += x2d
         ctx.add_residual = add_residual
-        ctx.save_for_backward(x2d, Y, O, lse, Mean, RSTD, masks, Wc, ln_w, ln_b, Wo)
+        ctx.save_for_backward(x2d, Y, O, lse, Mean, RSTD, masks, Wc, ln_w, ln_b, Wo, tiles)
         ctx.dims = (b, n, d, heads, dim_head, pad, transposed)
         ctx.has_bias = (bq is not None, bg is not None)
         return out.view(b, n, n, d)
@@ -168,7 +169,7 @@ class TriangleAttentionFunction(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dout):
-        x2d, Y, O, lse, Mean, RSTD, mask5, Wc, ln_w, ln_b, Wo = ctx.saved_tensors
+        x2d, Y, O, lse, Mean, RSTD, mask5, Wc, ln_w, ln_b, Wo, tiles = ctx.saved_tensors
         b, n, d, heads, dh, pad, transposed = ctx.dims
         inner = heads * dh
         M, Nt = Y.shape
@@ -184,7 +185,7 @@ class TriangleAttentionFunction(torch.autograd.Function):
         dO = dO.view(b, n, n, heads, dh)
         if transposed:
             dO, O = dO.transpose(1, 2), O.transpose(1, 2)
-        _, _, _, dbias = evoattention_backward(dO, Q, K, V, mask5, Bv, O, lse, True, out=(dQ, dK, dV))
+        _, _, _, dbias = evoattention_backward(dO, Q, K, V, mask5, Bv, O, lse, True, out=(dQ, dK, dV), bias_tiles=tiles)
         dBv[:, 0].copy_(dbias[:, 0])
         if pad:
             dY[:, 4 * inner + heads:].zero_()

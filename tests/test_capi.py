@@ -100,6 +100,14 @@ def test_attention_workspace_contract():
     bw = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
     assert bw >= 1 * 2 * 2 * 64 * 4                                      # at least delta
     assert lib.mf_evoattn_bwd(C.byref(a)) == -6
+    # tiles of the pair bias kept from the forward: the backward's workspace shrinks by exactly their size
+    tiles = lib.mf_evoattn_bias_tiles_bytes(C.byref(a))
+    assert tiles == need
+    a.bias_tiles_bwd = 0x30000
+    assert lib.mf_evoattn_bwd_workspace_bytes(C.byref(a)) == bw - tiles
+    a.workspace, a.workspace_bytes = 0x40000, bw
+    a.bias_tiles_bwd = 0x30008
+    assert lib.mf_evoattn_bwd(C.byref(a)) == -5 and "bias_tiles_bwd" in lib.mf_last_error().decode()
 
 
 def test_python_wrapper_fails_loudly_without_gpu_tensors():

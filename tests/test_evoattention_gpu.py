@@ -244,6 +244,34 @@ def test_no_bias_gradient_requested_and_function_signature():
         TritonEvoformer(dev["q"], dev["k"][..., :16], dev["v"], dev["mask"], dev["bias"])
 
 
+@pytest.mark.parametrize("B,N,S,H,D,nm,dtype,bias_dtype", [(1, 5, 100, 4, 32, 7, torch.bfloat16, torch.float32),
+                                                           (2, 3, 64, 2, 16, 0, torch.float16, torch.bfloat16),
+                                                           (1, 4, 72, 3, 64, 5, torch.float32, torch.float32)])
+def test_backward_reads_the_bias_tiles_the_forward_left(B, N, S, H, D, nm, dtype, bias_dtype):
+    """The forward can leave the pair bias in the backward's tile order (one preparation launch for both orders);
+    a backward given those tiles must return exactly what it returns after preparing its own copy, from a smaller
+    workspace, and the forward's own results must not depend on the option."""
+    import ctypes as C
+    from megafold_amd import _lib
+    inp = workloads.evoattention_inputs(B, N, S, H, D, nm, dtype=dtype, seed=21, bias_dtype=bias_dtype)
+    dev = to_dev(inp)
+    O1, lse1, saved1 = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"])
+    O2, lse2, saved2 = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"], save_bias_tiles=True)
+    assert len(saved1) == 5 and len(saved2) == 6
+    assert torch.equal(O1, O2) and torch.equal(lse1, lse2)
+    want = evoattention_backward(dev["dO"], *saved1, O1, lse1, True)
+    got = evoattention_backward(dev["dO"], *saved2[:5], O2, lse2, True, bias_tiles=saved2[5])
+    for w, g_ in zip(want, got):
+        assert torch.equal(w, g_)
+    a = _lib.EvoAttnArgs()
+    a.B, a.N, a.S, a.H, a.D = B, N, S, H, D
+    a.dtype = _lib.dtype_code(dtype)
+    a.dbias = 0x10000
+    full = _lib.lib().mf_evoattn_bwd_workspace_bytes(C.byref(a))
+    a.bias_tiles_bwd = 0x20000
+    assert full - _lib.lib().mf_evoattn_bwd_workspace_bytes(C.byref(a)) == _lib.lib().mf_evoattn_bias_tiles_bytes(C.byref(a)) == saved2[5].numel()
+
+
 def test_config5_peak_activation_memory():
     """C5 [1, 768, 768, 4, 32]: peak extra memory of fwd+bwd stays at the O(N*S*H*D) bound — O, dQ, dK,
     dV (144 MiB each) + LSE, delta, dBias (9 MiB each) — plus the declared workspace (the 9 MiB tiled copy of
