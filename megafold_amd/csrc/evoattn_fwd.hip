@@ -406,54 +406,53 @@ hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream) {
 }
 
 // ---- pair bias of any float dtype / strides -> tiled fp32 copy times `mult`, zero padded ------------
-// One thread writes one float4 of the layout described at EvoParams::bias: of the forward's order, of the
-// backward's, or (dst_bwd given beside a forward-order dst) of both in one launch.
-__device__ __forceinline__ void bias_prep_one(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj,
-                                              float* dst, int H, int S, int nt, float mult, bool backward_layout, int64_t idx) {
-  // thread -> float4 of the tile.  Backward layout: in storage order (a lane's four values come from
-  // four rows, consecutive lanes read consecutive keys).  Forward layout: eight consecutive threads
-  // take the 32 consecutive keys of one query row, so that both the reads (128 bytes per row) and the
-  // stores (adjacent chunks for adjacent rows) stay in runs.
-  int l, c4;
-  if (backward_layout) { l = (int)(idx & 63); c4 = (int)((idx >> 6) & 3); }
-  else { const int t = (int)(idx & 255); c4 = t & 3; l = 32 * ((t >> 2) & 1) + (t >> 3); }
-  const int64_t tile = idx >> 8;
-  const int t1 = (int)(tile % nt);
-  const int64_t r1 = tile / nt;
-  const int t0 = (int)(r1 % nt);
+// A work-group takes one 32 x 32 tile (query block ti, key block tj) of one (b, h): 8 threads read the 32
+// consecutive keys of a query row, the tile goes through LDS, and every thread writes one float4 of the layout
+// described at EvoParams::bias — of the forward's order (tile (ti, tj): lane = query, registers = keys), of the
+// backward's (tile (tj, ti): lane = key, registers = queries), or of both from the one read.
+__global__ void __launch_bounds__(256) bias_prep_kernel(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si,
+                                                        int64_t sj, float* dst_fwd, float* dst_bwd, int H, int S, int nt,
+                                                        float mult) {
+  __shared__ float tile[32][33];
+  const int t = threadIdx.x;
+  const int64_t tidx = blockIdx.x;
+  const int tj = (int)(tidx % nt);
+  const int64_t r1 = tidx / nt;
+  const int ti = (int)(r1 % nt);
   const int64_t bh = r1 / nt;
   const int h = (int)(bh % H);
   const int64_t b = bh / H;
-  const int x = l & 31, g = l >> 5;
-  f32x4 v;
+  {
+    const int r = t >> 3, c = (t & 7) * 4;
+    const int i = 32 * ti + r;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    // forward: tile (qt = t0, jt = t1); backward: tile (jt = t0, it = t1)
-    const int i = backward_layout ? 32 * t1 + 16 * g + 4 * c4 + e : 32 * t0 + x;
-    const int j = backward_layout ? 32 * t0 + x : 32 * t1 + 16 * g + 4 * c4 + e;
-    v[e] = (i < S && j < S) ? load_any(src, dtype, b * sb + h * sh + i * si + j * sj) * mult : 0.0f;
+    for (int e = 0; e < 4; ++e) {
+      const int j = 32 * tj + c + e;
+      tile[r][c + e] = (i < S && j < S) ? load_any(src, dtype, b * sb + h * sh + i * si + j * sj) * mult : 0.0f;
+    }
   }
-  *reinterpret_cast<f32x4*>(dst + tile * 1024 + 4 * (c4 * 64 + l)) = v;
-}
-
-__global__ void __launch_bounds__(256) bias_prep_kernel(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si,
-                                                        int64_t sj, float* dst, float* dst_bwd, int H, int S, int nt,
-                                                        float mult, int backward_layout, int64_t total4) {
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (int64_t)gridDim.x * 256) {
-    bias_prep_one(src, dtype, sb, sh, si, sj, dst, H, S, nt, mult, backward_layout != 0, idx);
-    if (dst_bwd) bias_prep_one(src, dtype, sb, sh, si, sj, dst_bwd, H, S, nt, mult, true, idx);
+  __syncthreads();
+  // float4 number t of a tile: lane l = t & 63 (x = l & 31, g = l >> 5), chunk c4 = t >> 6; value e is column / row
+  // 16 g + 4 c4 + e against row / column x
+  const int l = t & 63, c4 = t >> 6, x = l & 31, g = l >> 5, k0 = 16 * g + 4 * c4;
+  if (dst_fwd) {
+    const f32x4 v = {tile[x][k0], tile[x][k0 + 1], tile[x][k0 + 2], tile[x][k0 + 3]};
+    *reinterpret_cast<f32x4*>(dst_fwd + ((bh * nt + ti) * nt + tj) * 1024 + 4 * t) = v;
+  }
+  if (dst_bwd) {
+    const f32x4 v = {tile[k0][x], tile[k0 + 1][x], tile[k0 + 2][x], tile[k0 + 3][x]};
+    *reinterpret_cast<f32x4*>(dst_bwd + ((bh * nt + tj) * nt + ti) * 1024 + 4 * t) = v;
   }
 }
 
 hipError_t launch_bias_prep(const void* src, int dtype, int64_t sb, int64_t sh, int64_t si, int64_t sj, float* dst,
                             int B, int H, int S, float mult, bool backward_layout, hipStream_t stream, float* dst_bwd) {
   const int nt = (S + 31) / 32;
-  const int64_t total4 = (int64_t)B * H * nt * nt * 256;
-  if (total4 == 0) return hipSuccess;
-  int64_t blocks = (total4 + 255) / 256;
-  if (blocks > 8192) blocks = 8192;
-  hipLaunchKernelGGL(bias_prep_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dtype, sb, sh, si, sj, dst,
-                     dst_bwd, H, S, nt, mult, backward_layout ? 1 : 0, total4);
+  const int64_t tiles = (int64_t)B * H * nt * nt;
+  if (tiles == 0) return hipSuccess;
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(bias_prep_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, src, dtype, sb, sh, si, sj,
+                     backward_layout ? nullptr : dst, backward_layout ? dst : dst_bwd, H, S, nt, mult);
   return hipGetLastError();
 }
 
