@@ -63,6 +63,8 @@ PWA_CASES = [
     (2, 5, 37, 64, 128, 8, 32, 0, torch.bfloat16),           # ragged tiles, no mask, batch of two
     (1, 7, 77, 32, 64, 2, 16, 9, torch.float16),
     (1, 6, 40, 64, 128, 4, 32, 3, torch.float32),
+    (1, 9, 200, 64, 128, 8, 32, 11, torch.bfloat16),         # 14 key tiles of 16: the middle instantiation of the kernel
+    (1, 6, 70, 64, 128, 8, 32, 4, torch.float16),            # the dedicated kernels in fp16
 ]
 
 
@@ -101,6 +103,8 @@ OPM_CASES = [
     (2, 5, 37, 64, 32, 128, False, False, torch.bfloat16),
     (1, 7, 33, 32, 8, 64, True, False, torch.float16),
     (1, 6, 40, 64, 16, 128, True, True, torch.float32),
+    (1, 9, 52, 64, 32, 128, True, True, torch.float16),      # the fused kernels in fp16
+    (2, 20, 26, 64, 32, 128, True, False, torch.bfloat16),   # ragged position tiles in both directions, batch of two
 ]
 
 
