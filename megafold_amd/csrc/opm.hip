@@ -348,12 +348,14 @@ __global__ void __launch_bounds__(256) opm_dw_reduce_kernel(const OpmDwParams p)
 //               registers (A operand), dOut rows from LDS; laid into LDS as pair rows of 512 values
 //   stage B     wavefront (rt, sh): rows (2 positions o, 16 f) x 64 values s, contraction over (t, h) = 128:
 //               dO rows as plain fragments, the operand rows through transposing LDS reads
-// The tile's 128 operand rows and 32 dOut rows arrive by direct loads, double buffered.
+// The tile's 128 operand rows and 32 dOut rows arrive by direct loads, double buffered, and so is the dO tile: between
+// two barriers the work-group runs stage B of job j and stage A of job j + 1, whose chains are independent (one
+// barrier per job, and each stage covers the LDS latencies of the other).
 constexpr int DAB_OSTR = 1024 + 16;             // bytes between pair rows of the dO tile
 constexpr int DAB_LDS_P = 0;                    // two tiles of 128 operand rows x 256 bytes
 constexpr int DAB_LDS_D = 2 * 32768;            // two tiles of 32 dOut rows x 256 bytes
 constexpr int DAB_LDS_O = DAB_LDS_D + 2 * 8192;
-constexpr int DAB_LDS_BYTES = DAB_LDS_O + 32 * DAB_OSTR;
+constexpr int DAB_LDS_BYTES = DAB_LDS_O + 2 * 32 * DAB_OSTR;   // two dO tiles
 
 struct OpmDabParams {
   int B, n, tiles_t, units_per_batch, jobs, per_group, groups, transposed;
@@ -387,7 +389,7 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
     fh = u & 1;
   };
   // direct loads of a job's tiles: LDS row r, 16-byte position pos holds chunk pos ^ (r & 15) of the row
-  auto issue = [&](int job, int buf) {
+  auto issue_p = [&](int job, int buf) {           // the 128 operand rows
     int bb, o0, fh, t0;
     decode(job, bb, o0, fh, t0);
     const char* pbase = reinterpret_cast<const char*>(p.opnd) + (int64_t)bb * n * 32 * 256;
@@ -398,6 +400,10 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
       grow = grow < n * 32 ? grow : n * 32 - 1;
       dma16((unsigned)(grow * 256 + ((pos ^ (row & 15)) << 4)), pbase, lds0 + DAB_LDS_P + buf * 32768 + rd * 8192 + wv * 1024);
     }
+  };
+  auto issue_d = [&](int job, int buf) {           // the 32 dOut rows
+    int bb, o0, fh, t0;
+    decode(job, bb, o0, fh, t0);
     const int r = t512 >> 4, pos = t512 & 15;
     int o = o0 + (r >> 2), t = t0 + (r & 3);
     o = o < n ? o : n - 1;
@@ -407,7 +413,6 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
     dma16((unsigned)(pair * 256 + ((pos ^ (r & 15)) << 4)), dbase, lds0 + DAB_LDS_D + buf * 8192 + wv * 1024);
   };
 
-  unsigned char* Ob = smem + DAB_LDS_O;
   frag wf[2][8];
   f32x16 acc[2] = {acc_zero(), acc_zero()};
   int cur_unit = -1, cur_fh = -1, piece = 0;
@@ -419,12 +424,80 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
       for (int r = 0; r < 16; ++r)
         dst[(rt * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + sh * 64 + c * 32 + x] = acc[c][r];
   };
-
-  issue(j_begin, 0);
-  for (int job = j_begin; job < j_end; ++job) {
-    const int buf = (job - j_begin) & 1;
+  // rows f * 32 + h of wt for this wavefront's two values f, h permuted so that a register holds 16 g + r
+  auto load_wf = [&](int fh) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const T* wrow = reinterpret_cast<const T*>(p.wt) + (int64_t)((fh * 16 + 2 * wv + a) * 32 + unperm32(x)) * 128 + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) wf[a][ks] = ld8<T>(wrow + 16 * ks);
+    }
+    cur_fh = fh;
+  };
+  // stage A of a job: dO rows of the tile's 32 pairs into dO tile `ob`
+  auto stage_a = [&](int job, int db, int ob) {
     int bb, o0, fh, t0;
     decode(job, bb, o0, fh, t0);
+    if (fh != cur_fh) {
+      load_wf(fh);
+      wait_vm<0>();
+    }
+    const unsigned char* Dt = smem + DAB_LDS_D + db * 8192;
+    f32x16 o[2] = {acc_zero(), acc_zero()};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const frag df = ld8<T>(reinterpret_cast<const T*>(Dt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
+      o[0] = mma(wf[0][ks], df, o[0]);             // rows = h (16 g + r in register r), columns = pairs
+      o[1] = mma(wf[1][ks], df, o[1]);
+    }
+    const bool live = t0 + (x & 3) < n;            // pairs past the edge contribute nothing
+    unsigned char* orow = smem + DAB_LDS_O + ob * 32 * DAB_OSTR + x * DAB_OSTR;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int q = 4 * (2 * wv + a) + 2 * g + u;            // 16-byte chunk (f_local * 32 + 16 g + 8 u) / 8
+        st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), live ? acc_half<T>(o[a], u) : frag_zero<T>());
+      }
+  };
+  // stage B of a job: its dO tile `ob` against its operand rows `pb`
+  auto stage_b = [&](int pb, int ob) {
+    const unsigned char* Pt = smem + DAB_LDS_P + pb * 32768;
+    const unsigned char* Ob = smem + DAB_LDS_O + ob * 32 * DAB_OSTR;
+    const int a4 = (l >> 2) & 3;
+    const int ol = 2 * rt + (x >> 4), fl = x & 15;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const int q = 4 * fl + 2 * (ks & 1) + g;
+      const frag of = ld8<T>(reinterpret_cast<const T*>(Ob + (ol * 4 + (ks >> 1)) * DAB_OSTR + ((q ^ ((q >> 4) & 3)) << 4)));
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int col = sh * 64 + c * 32 + plain_chunk(l);
+        const int r0 = 16 * ks + 8 * g + a4, r1 = r0 + 4;
+        const unsigned char* p0 = Pt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
+        const unsigned char* p1 = Pt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        s16x8 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+        acc[c] = mma(of, __builtin_bit_cast(frag, v), acc[c]);   // rows = (o, f), columns = s
+      }
+    }
+  };
+
+  // prologue: the first job's tiles and the second job's dOut rows, then stage A of the first job
+  issue_d(j_begin, 0);
+  issue_p(j_begin, 0);
+  if (j_begin + 1 < j_end) issue_d(j_begin + 1, 1);
+  wait_vm<0>();
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  stage_a(j_begin, 0, 0);
+  for (int job = j_begin; job < j_end; ++job) {
+    const int k = (job - j_begin) & 1;
     const int unit = job / p.tiles_t;
     if (unit != cur_unit) {
       if (cur_unit >= 0) {
@@ -433,67 +506,15 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
         acc[0] = acc_zero(); acc[1] = acc_zero();
       }
       cur_unit = unit;
-      if (fh != cur_fh) {                          // rows f * 32 + h of wt, h permuted so that a register holds 16 g + r
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const T* wrow = reinterpret_cast<const T*>(p.wt) + (int64_t)((fh * 16 + 2 * wv + a) * 32 + unperm32(x)) * 128 + 8 * g;
-#pragma unroll
-          for (int ks = 0; ks < 8; ++ks) wf[a][ks] = ld8<T>(wrow + 16 * ks);
-        }
-        cur_fh = fh;
-      }
     }
-    wait_vm<0>();                                  // this job's rows (and wt) have arrived
+    wait_vm<0>();                                  // operand rows of this job, dOut rows of the next have arrived
     __builtin_amdgcn_s_waitcnt(0xC07F);
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    if (job + 1 < j_end) issue(job + 1, buf ^ 1);
-    // ---- stage A
-    {
-      const unsigned char* Dt = smem + DAB_LDS_D + buf * 8192;
-      f32x16 o[2] = {acc_zero(), acc_zero()};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const frag df = ld8<T>(reinterpret_cast<const T*>(Dt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
-        o[0] = mma(wf[0][ks], df, o[0]);           // rows = h (16 g + r in register r), columns = pairs
-        o[1] = mma(wf[1][ks], df, o[1]);
-      }
-      const bool live = t0 + (x & 3) < n;          // pairs past the edge contribute nothing
-      unsigned char* orow = Ob + x * DAB_OSTR;
-#pragma unroll
-      for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const int q = 4 * (2 * wv + a) + 2 * g + u;          // 16-byte chunk (f_local * 32 + 16 g + 8 u) / 8
-          st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), live ? acc_half<T>(o[a], u) : frag_zero<T>());
-        }
-    }
-    barrier_keep_vm<63>();                         // LDS hand-over only: the next job's rows keep travelling
-    // ---- stage B
-    {
-      const unsigned char* Pt = smem + DAB_LDS_P + buf * 32768;
-      const int a4 = (l >> 2) & 3;
-      const int ol = 2 * rt + (x >> 4), fl = x & 15;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const int q = 4 * fl + 2 * (ks & 1) + g;
-        const frag of = ld8<T>(reinterpret_cast<const T*>(Ob + (ol * 4 + (ks >> 1)) * DAB_OSTR + ((q ^ ((q >> 4) & 3)) << 4)));
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const int col = sh * 64 + c * 32 + plain_chunk(l);
-          const int r0 = 16 * ks + 8 * g + a4, r1 = r0 + 4;
-          const unsigned char* p0 = Pt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
-          const unsigned char* p1 = Pt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
-          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
-          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
-          typedef short s16x8 __attribute__((ext_vector_type(8)));
-          s16x8 v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
-          acc[c] = mma(of, __builtin_bit_cast(frag, v), acc[c]);   // rows = (o, f), columns = s
-        }
-      }
-    }
+    __builtin_amdgcn_s_barrier();                  // ... for every wavefront, and this job's dO tile is complete; the
+    asm volatile("" ::: "memory");                 // buffers requested below were last read before this barrier
+    if (job + 1 < j_end) issue_p(job + 1, k ^ 1);
+    if (job + 2 < j_end) issue_d(job + 2, k);
+    if (job + 1 < j_end) stage_a(job + 1, k ^ 1, k ^ 1);
+    stage_b(k, k);
   }
   flush(piece);
 }
