@@ -484,6 +484,43 @@ def main():
             "protocol": "same step, 100 warm-up + 200 timed, run in this process after the timed region"},
         "hbm_GBps_at_algorithmic_bytes": round(468.0 / ms_per_step, 1),
     }
+    if not args.no_extras:
+        # the memory-lean order of the backward (opt-in, MF_EVO_BWD_LEAN): same step, 100 warm-up + 200 timed, and its
+        # peak activation memory through the autograd operator
+        from megafold_amd.model.FusedEvoAttention import evoattention as ev
+
+        def lean_step():
+            O, lse, (Q, K_, V, mask, bias_, tiles) = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"],
+                                                                          dev["bias"], save_bias_tiles=True)
+            evoattention_backward(dev["dO"], Q, K_, V, mask, bias_, O, lse, True, bias_tiles=tiles, lean=True)
+
+        for _ in range(100):
+            lean_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            lean_step()
+        torch.cuda.synchronize()
+        lean_ms = (time.perf_counter() - t0) * 1e3 / 200
+        q, k, v = (dev[n].clone().requires_grad_() for n in "qkv")
+        bias = dev["bias"].clone().requires_grad_()
+        ev.MEMORY_LEAN = True
+        try:
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            out = TritonEvoformer(q, k, v, dev["mask"], bias)
+            out.backward(dev["dO"])
+            torch.cuda.synchronize()
+            lean_peak = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+        finally:
+            ev.MEMORY_LEAN = False
+        del out, q, k, v, bias
+        res["memory_lean_order"] = {"ms_per_step": round(lean_ms, 5), "value": round(fl["total"] / lean_ms / 1e9, 2),
+                                    "peak_act_mib": round(lean_peak, 2),
+                                    "note": "opt-in: bias gradient before dQ/dK/dV, its partial sums in the dQ buffer, "
+                                            "delta from its own kernel"}
     if args.calibrate_copy:
         src = torch.empty(256 * 2 ** 20, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)

@@ -80,6 +80,13 @@ const char* mf_last_error(void);
 #define MF_EVO_BWD_DQKV 1
 #define MF_EVO_BWD_DBIAS 2
 #define MF_EVO_BWD_PREP 4
+/* Modifier bit: memory-lean order.  The bias gradient runs BEFORE dq, dk, dv: rowsum(dO * o) comes from a kernel of
+ * its own and the partial sums of the bias gradient live in the dq buffer, which nothing has written yet, instead of
+ * in the workspace (smaller workspace: query it with this bit set).  Costs one more pass over dO and o.  Needs
+ * dbias != NULL, a contiguous dq ([B, N, S, H, D]) and a dq buffer at least as large as the partial sums
+ * (mf_evoattn_bwd_lean_ok reports both; MF_ERR_SHAPE otherwise).  With split phases the order of the calls is PREP,
+ * DBIAS, DQKV, each with this bit. */
+#define MF_EVO_BWD_LEAN 8
 
 typedef struct mf_evoattn_args {
   int32_t B, N, S, H, D;
@@ -114,6 +121,7 @@ typedef struct mf_evoattn_args {
 uint64_t mf_evoattn_fwd_workspace_bytes(const mf_evoattn_args* a);
 uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a);
 uint64_t mf_evoattn_bias_tiles_bytes(const mf_evoattn_args* a);
+int mf_evoattn_bwd_lean_ok(const mf_evoattn_args* a); /* 1 if MF_EVO_BWD_LEAN can be used with these arguments */
 int mf_evoattn_fwd(const mf_evoattn_args* a);
 int mf_evoattn_bwd(const mf_evoattn_args* a);
 

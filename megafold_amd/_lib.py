@@ -14,7 +14,7 @@ LIB_PATH = PKG / "lib" / "libmegafold_amd.so"
 
 MF_F32, MF_F16, MF_BF16, MF_BOOL = 0, 1, 2, 3
 MF_ACT_NONE, MF_ACT_SWIGLU = 0, 1
-MF_EVO_BWD_DQKV, MF_EVO_BWD_DBIAS, MF_EVO_BWD_PREP = 1, 2, 4
+MF_EVO_BWD_DQKV, MF_EVO_BWD_DBIAS, MF_EVO_BWD_PREP, MF_EVO_BWD_LEAN = 1, 2, 4, 8
 
 I64x4 = C.c_int64 * 4
 I64x3 = C.c_int64 * 3
@@ -88,6 +88,7 @@ SYMBOLS = {
     "mf_evoattn_fwd_workspace_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_bwd_workspace_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_bias_tiles_bytes": (C.c_uint64, [C.POINTER(EvoAttnArgs)]),
+    "mf_evoattn_bwd_lean_ok": (C.c_int, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_fwd": (C.c_int, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_bwd": (C.c_int, [C.POINTER(EvoAttnArgs)]),
     "mf_evoattn_fwd_noalloc": (C.c_int, [C.POINTER(EvoAttnArgs)]),

@@ -15,7 +15,7 @@ namespace {
 
 struct Plan {
   int bias_nt;              // 32 x 32 tiles per side of the fp32 bias/scale copy the kernels read
-  uint64_t off_bias, off_delta, off_part, dq_scratch_bytes, total;
+  uint64_t off_bias, off_delta, off_part, dq_scratch_bytes, part_bytes, total;
   int n_chunks, rows_per_chunk;
 };
 
@@ -39,7 +39,10 @@ Plan make_plan(const mf_evoattn_args* a, bool backward) {
       // the first chunk writes into dbias itself
       if (pl.n_chunks > 1) part_bytes = (uint64_t)(pl.n_chunks - 1) * a->B * a->H * a->S * a->S * 4;
     }
-    // the multi-pass dQ array of the dQ/dK/dV kernel is dead before the bias-gradient kernel starts: one region
+    // the multi-pass dQ array of the dQ/dK/dV kernel is dead before the bias-gradient kernel starts: one region.
+    // In the memory-lean order the partial sums live in the dq buffer instead.
+    pl.part_bytes = part_bytes;
+    if (a->dbias && (a->phases & MF_EVO_BWD_LEAN)) part_bytes = 0;
     pl.dq_scratch_bytes = evo_bwd_dqkv_pw_scratch_bytes(a->dtype, a->S, a->D, evo_num_cu());
     off += align256(part_bytes > pl.dq_scratch_bytes ? part_bytes : pl.dq_scratch_bytes);
   }
@@ -131,6 +134,21 @@ extern "C" uint64_t mf_evoattn_bias_tiles_bytes(const mf_evoattn_args* a) {
   const uint64_t nt = ((uint64_t)a->S + 31) / 32;
   return align256((uint64_t)a->B * a->H * nt * nt * 4096);
 }
+namespace {
+// The memory-lean order keeps the bias gradient's partial sums in the dq buffer: it must be one contiguous
+// [B, N, S, H, D] array and large enough.
+bool lean_ok(const mf_evoattn_args* a, const Plan& pl) {
+  if (!a->dbias || !a->dq) return false;
+  const int64_t D = a->D, H = a->H, S = a->S, N = a->N;
+  if (a->dq_stride[3] != D || a->dq_stride[2] != H * D || a->dq_stride[1] != S * H * D || a->dq_stride[0] != N * S * H * D)
+    return false;
+  return pl.part_bytes <= (uint64_t)a->B * N * S * H * D * dtype_size(a->dtype);
+}
+}  // namespace
+extern "C" int mf_evoattn_bwd_lean_ok(const mf_evoattn_args* a) {
+  if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0 || dtype_size(a->dtype) == 0) return 0;
+  return lean_ok(a, make_plan(a, true)) ? 1 : 0;
+}
 extern "C" uint64_t mf_evoattn_bwd_workspace_bytes(const mf_evoattn_args* a) {
   if (!a || a->B <= 0 || a->N <= 0 || a->S <= 0 || a->H <= 0 || a->D <= 0) return 0;
   return make_plan(a, true).total;
@@ -216,14 +234,20 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
   if ((rc = check_tensor("dk", a->dk, a->dk_stride, es))) return rc;
   if ((rc = check_tensor("dv", a->dv, a->dv_stride, es))) return rc;
   if (a->dbias && !aligned16(a->dbias)) return fail(MF_ERR_ALIGN, "dbias is not 16-byte aligned");
-  if (a->phases < 0 || a->phases > (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS | MF_EVO_BWD_PREP)) return fail(MF_ERR_SHAPE, "phases %d unknown", a->phases);
+  if (a->phases < 0 || a->phases > (MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS | MF_EVO_BWD_PREP | MF_EVO_BWD_LEAN))
+    return fail(MF_ERR_SHAPE, "phases %d unknown", a->phases);
   const Plan pl = make_plan(a, true);
+  const bool lean = (a->phases & MF_EVO_BWD_LEAN) != 0;
+  if (lean && !lean_ok(a, pl))
+    return fail(MF_ERR_SHAPE, "MF_EVO_BWD_LEAN needs dbias, a contiguous dq and a dq buffer of at least %llu bytes "
+                "(see mf_evoattn_bwd_lean_ok)", (unsigned long long)pl.part_bytes);
   if (!a->workspace || a->workspace_bytes < pl.total)
     return fail(MF_ERR_WORKSPACE, "backward needs %llu workspace bytes, got %llu", (unsigned long long)pl.total,
                 (unsigned long long)(a->workspace ? a->workspace_bytes : 0));
   if (!aligned16(a->workspace)) return fail(MF_ERR_ALIGN, "workspace is not 16-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
-  const int phases = a->phases == 0 ? (MF_EVO_BWD_PREP | MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : a->phases;
+  const int which = a->phases & ~MF_EVO_BWD_LEAN;
+  const int phases = which == 0 ? (MF_EVO_BWD_PREP | MF_EVO_BWD_DQKV | MF_EVO_BWD_DBIAS) : which;
   EvoParams p;
   rc = fill_params(a, pl, p, stream, (phases & MF_EVO_BWD_PREP) != 0, true);
   if (rc) return rc;
@@ -238,13 +262,19 @@ extern "C" int mf_evoattn_bwd(const mf_evoattn_args* a) {
     const char* f = getenv("MF_TL_BLOCK"); p.tl_block = f ? atoi(f) : 0; }
 #endif
   p.rows_per_chunk = pl.rows_per_chunk;
-  p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
+  p.dbias_part = pl.n_chunks > 1 ? reinterpret_cast<float*>(lean ? a->dq : ws + pl.off_part) : nullptr;
   p.dq_scratch = pl.dq_scratch_bytes ? reinterpret_cast<float*>(ws + pl.off_part) : nullptr;
   hipError_t e = hipSuccess;
+  if (lean && (phases & MF_EVO_BWD_DBIAS)) {      // bias gradient first: its partial sums are in the dq buffer
+    e = launch_evo_delta(p, stream);
+    if (e != hipSuccess) return (int)e;
+    e = launch_evo_bwd_dbias(p, stream);
+    if (e != hipSuccess) return (int)e;
+  }
   if (phases & MF_EVO_BWD_DQKV) {
     e = launch_evo_bwd_dqkv(p, stream);
     if (e != hipSuccess) return (int)e;
   }
-  if ((phases & MF_EVO_BWD_DBIAS) && a->dbias) e = launch_evo_bwd_dbias(p, stream);
+  if (!lean && (phases & MF_EVO_BWD_DBIAS) && a->dbias) e = launch_evo_bwd_dbias(p, stream);
   return (int)e;
 }

@@ -55,6 +55,7 @@ struct EvoParams {
 hipError_t launch_evo_fwd(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dqkv(const EvoParams& p, hipStream_t stream);
 hipError_t launch_evo_bwd_dbias(const EvoParams& p, hipStream_t stream);
+hipError_t launch_evo_delta(const EvoParams& p, hipStream_t stream);   // p.delta = rowsum(dO * O) by its own kernel
 // Bias-gradient kernel that streams its rows through an LDS ring with direct loads (16-bit, D = 32, paired heads;
 // evoattn_bwd_dbias_ring.hip): whether it handles the problem, and its launcher (same grid and chunking as
 // the paired-head form of evo_bwd_dbias_kernel; the caller sums the partial buffers).

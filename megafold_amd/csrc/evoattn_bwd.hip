@@ -1224,6 +1224,46 @@ template <typename T> static hipError_t launch_dbias_s(const EvoParams& p, hipSt
   return hipErrorInvalidValue;
 }
 
+// delta[b, n, h, s] = sum_d dO[b, n, s, h, d] O[b, n, s, h, d] on its own (evoattention.py:272-301): D / 8 lanes per
+// (s, h), consecutive lanes on consecutive 16-byte chunks of a position's H * D values.  The dQ/dK/dV kernels form
+// delta themselves; this kernel serves the order in which the bias gradient runs before them.
+template <typename T>
+__global__ void __launch_bounds__(256) evo_delta_kernel(const EvoParams p) {
+  const int CPR = p.D / 8;                                   // lanes per (s, h): 1, 2, 4 or 8
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)p.B * p.N * p.S * p.H * CPR;
+  const int64_t it = item < total ? item : total - 1;        // whole groups stay together: no early exit
+  const int dc = (int)(it % CPR);
+  int64_t r = it / CPR;
+  const int h = (int)(r % p.H); r /= p.H;
+  const int s = (int)(r % p.S); r /= p.S;
+  const int n = (int)(r % p.N);
+  const int64_t b = r / p.N;
+  const T* dO = reinterpret_cast<const T*>(p.dO.ptr) + b * p.dO.sb + n * p.dO.sn + s * p.dO.ss + h * p.dO.sh + 8 * dc;
+  const T* O = reinterpret_cast<const T*>(p.o.ptr) + b * p.o.sb + n * p.o.sn + s * p.o.ss + h * p.o.sh + 8 * dc;
+  const frag_t<T> a = ld8<T>(dO), c = ld8<T>(O);
+  float part = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)c[e];
+  if (CPR >= 2) part += __shfl_xor(part, 1);
+  if (CPR >= 4) part += __shfl_xor(part, 2);
+  if (CPR >= 8) part += __shfl_xor(part, 4);
+  if (dc == 0 && item < total) p.delta[((b * p.N + n) * p.H + h) * p.S + s] = part;
+}
+
+hipError_t launch_evo_delta(const EvoParams& p, hipStream_t stream) {
+  const int64_t total = (int64_t)p.B * p.N * p.S * p.H * (p.D / 8);
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  switch (p.dtype) {
+    case MF_BF16: hipLaunchKernelGGL(evo_delta_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, p); break;
+    case MF_F16: hipLaunchKernelGGL(evo_delta_kernel<f16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, p); break;
+    case MF_F32: hipLaunchKernelGGL(evo_delta_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 hipError_t launch_evo_bwd_dbias(const EvoParams& p, hipStream_t stream) {
   switch (p.dtype) {
     case MF_BF16: return launch_dbias_s<bf16_t>(p, stream);

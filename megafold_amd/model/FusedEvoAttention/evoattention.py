@@ -32,6 +32,10 @@ import torch
 
 from ... import _lib
 
+# Default of evoattention_backward's ``lean``: trade one more pass over dO and O for a workspace without the bias
+# gradient's partial sums (peak activation memory inside the O(N S H D) bound + the bias tiles).
+MEMORY_LEAN = False
+
 __all__ = ["EvoformerAttention", "TritonEvoformer", "evoattention_forward", "evoattention_backward",
            "evoattention_forward_noalloc"]
 
@@ -152,13 +156,17 @@ def evoattention_forward_noalloc(Q, K, V, res_mask, pair_bias, O, lse) -> None:
         _lib.check(_lib.lib().mf_evoattn_fwd_noalloc(C.byref(a)), "mf_evoattn_fwd_noalloc")
 
 
-def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None, out=None, bias_tiles=None):
+def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phase_hook=None, out=None, bias_tiles=None,
+                          lean=None):
     """dQ, dK, dV, dBias(fp32 [B, 1, H, S, S] or None) from the saved forward state.
 
     ``out = (dQ, dK, dV)``, if given, are the tensors to write (``[B, N, S, H, D]`` in Q's dtype, unit
     stride on D and 16-byte multiples elsewhere, e.g. column slices of a wider matrix); otherwise
     contiguous tensors are allocated.  ``bias_tiles``: the sixth saved tensor of
-    ``evoattention_forward(..., save_bias_tiles=True)`` for the same inputs.
+    ``evoattention_forward(..., save_bias_tiles=True)`` for the same inputs.  ``lean`` (default: the module-level
+    ``MEMORY_LEAN``): the memory-lean order of ``MF_EVO_BWD_LEAN`` where the library can use it (bias gradient wanted,
+    contiguous dQ large enough for its partial sums) — the bias gradient runs first with its partial sums in the dQ
+    buffer, at the price of one more pass over dO and O.
 
     ``phase_hook(name)``, if given, is called before and after each backward phase ("prep", "dqkv",
     "dbias"), which are then enqueued by separate C-ABI calls (used by the benchmark to bracket each
@@ -189,6 +197,9 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phas
         a.dv_stride = _lib.I64x4(*dV.stride()[:4])
         if bias_tiles is not None:
             a.bias_tiles_bwd = bias_tiles.data_ptr()
+        lean = MEMORY_LEAN if lean is None else lean
+        lean_bit = _lib.MF_EVO_BWD_LEAN if (lean and dbias is not None and lib.mf_evoattn_bwd_lean_ok(C.byref(a))) else 0
+        a.phases = lean_bit
         nbytes = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=Q.device)
         a.workspace = ws.data_ptr()
@@ -196,11 +207,13 @@ def evoattention_backward(dO, Q, K, V, mask, bias, O, lse, need_dbias=True, phas
         if phase_hook is None:
             _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd")
         else:
-            for name, bit in (("prep", _lib.MF_EVO_BWD_PREP), ("dqkv", _lib.MF_EVO_BWD_DQKV),
-                              ("dbias", _lib.MF_EVO_BWD_DBIAS)):
+            order = (("prep", _lib.MF_EVO_BWD_PREP), ("dqkv", _lib.MF_EVO_BWD_DQKV), ("dbias", _lib.MF_EVO_BWD_DBIAS))
+            if lean_bit:
+                order = (order[0], order[2], order[1])
+            for name, bit in order:
                 if bit == _lib.MF_EVO_BWD_DBIAS and dbias is None:
                     continue
-                a.phases = bit
+                a.phases = bit | lean_bit
                 phase_hook(name)
                 _lib.check(lib.mf_evoattn_bwd(C.byref(a)), "mf_evoattn_bwd[%s]" % name)
                 phase_hook(name)

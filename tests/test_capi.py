@@ -110,6 +110,35 @@ def test_attention_workspace_contract():
     assert lib.mf_evoattn_bwd(C.byref(a)) == -5 and "bias_tiles_bwd" in lib.mf_last_error().decode()
 
 
+def test_attention_memory_lean_contract():
+    """MF_EVO_BWD_LEAN keeps the bias gradient's partial sums in the dq buffer: accepted only with dbias, a contiguous dq
+    and a dq buffer that can hold them; the workspace query with the bit set leaves the partial sums out."""
+    lib = _lib.lib()
+    a = _evo_args()
+    a.N, a.S = 64, 128                                   # 64 rows: several row chunks, dq larger than the partial sums
+    B, N, S, H, D = a.B, a.N, a.S, a.H, a.D
+    std = _lib.I64x4(N * S * H * D, S * H * D, H * D, D)
+    a.q_stride = a.k_stride = a.v_stride = a.o_stride = std
+    for f in ("dO", "dq", "dk", "dv", "dbias"):
+        setattr(a, f, 0x10000)
+    a.do_stride = a.dq_stride = a.dk_stride = a.dv_stride = std
+    full = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
+    assert lib.mf_evoattn_bwd_lean_ok(C.byref(a)) == 1
+    a.phases = _lib.MF_EVO_BWD_LEAN
+    lean = lib.mf_evoattn_bwd_workspace_bytes(C.byref(a))
+    assert lean < full
+    a.workspace, a.workspace_bytes = 0x40000, lean
+    a.dq_stride = _lib.I64x4(N * S * H * 2 * D, S * H * 2 * D, H * 2 * D, 2 * D)      # a column slice of a wider matrix
+    assert lib.mf_evoattn_bwd_lean_ok(C.byref(a)) == 0
+    assert lib.mf_evoattn_bwd(C.byref(a)) == -2 and "MF_EVO_BWD_LEAN" in lib.mf_last_error().decode()
+    a.dq_stride = std
+    a.dbias = None
+    assert lib.mf_evoattn_bwd_lean_ok(C.byref(a)) == 0
+    a.dbias = 0x10000
+    a.phases = 16
+    assert lib.mf_evoattn_bwd(C.byref(a)) == -2 and "phases" in lib.mf_last_error().decode()
+
+
 def test_python_wrapper_fails_loudly_without_gpu_tensors():
     import torch
     from megafold_amd.model.FusedEvoAttention.evoattention import TritonEvoformer

@@ -272,6 +272,64 @@ def test_backward_reads_the_bias_tiles_the_forward_left(B, N, S, H, D, nm, dtype
     assert full - _lib.lib().mf_evoattn_bwd_workspace_bytes(C.byref(a)) == _lib.lib().mf_evoattn_bias_tiles_bytes(C.byref(a)) == saved2[5].numel()
 
 
+@pytest.mark.parametrize("B,N,S,H,D,nm,dtype", [(1, 24, 100, 4, 32, 7, torch.bfloat16), (2, 9, 64, 2, 16, 0, torch.float16),
+                                                 (1, 40, 72, 3, 64, 5, torch.float32), (1, 300, 416, 4, 32, 20, torch.bfloat16)])
+def test_memory_lean_order_matches_the_default_order(B, N, S, H, D, nm, dtype):
+    """MF_EVO_BWD_LEAN: delta from its own kernel, the bias gradient before dQ/dK/dV with its partial sums in the dQ
+    buffer.  dQ, dK, dV come from the same kernel on the same inputs and must be identical; the bias gradient sees a
+    delta summed in another order and must agree to fp32 rounding; the workspace must be smaller by the partial sums."""
+    import ctypes as C
+    from megafold_amd import _lib
+    inp = workloads.evoattention_inputs(B, N, S, H, D, nm, dtype=dtype, seed=33)
+    dev = to_dev(inp)
+    O, lse, saved = evoattention_forward(dev["q"], dev["k"], dev["v"], dev["mask"], dev["bias"])
+    want = evoattention_backward(dev["dO"], *saved, O, lse, True, lean=False)
+    got = evoattention_backward(dev["dO"], *saved, O, lse, True, lean=True)
+    for w, g_ in zip(want[:3], got[:3]):
+        assert torch.equal(w, g_)
+    scale = float(want[3].abs().max())
+    assert float((want[3] - got[3]).abs().max()) <= 2e-5 * max(scale, 1.0)
+    calls = []
+    got2 = evoattention_backward(dev["dO"], *saved, O, lse, True, lean=True, phase_hook=calls.append)   # split phases
+    # the order is taken where dQ can hold the partial sums (the wrapper asks mf_evoattn_bwd_lean_ok); small dQ buffers
+    # keep the default order
+    assert calls[::2] in (["prep", "dbias", "dqkv"], ["prep", "dqkv", "dbias"])
+    if (N, S) in ((300, 416), (40, 72)):
+        assert calls[::2] == ["prep", "dbias", "dqkv"]
+    for a_, b_ in zip(got, got2):
+        assert torch.equal(a_, b_)
+    # a strided dQ cannot hold the partial sums: the library says so and the wrapper keeps the default order
+    wide = torch.empty((B, N, S, H, 2 * D), dtype=dtype, device="cuda")
+    outs = (wide[..., :D], torch.empty_like(O), torch.empty_like(O))
+    got3 = evoattention_backward(dev["dO"], *saved, O, lse, True, lean=True, out=outs)
+    for w, g_ in zip(want, got3):
+        assert torch.equal(w, g_)
+
+
+def test_config2_memory_lean_peak_activation():
+    """C2 with the memory-lean order: the peak of forward + backward stays within the O(N S H D) bound (150.75 MiB) plus the
+    tiled copies of the pair bias (two of 2.25 MiB: the forward's and the one kept for the backward)."""
+    from megafold_amd.model.FusedEvoAttention import evoattention as ev
+    dev = to_dev(workloads.config2())
+    q, k, v = (dev[n_].requires_grad_() for n_ in "qkv")
+    bias = dev["bias"].requires_grad_()
+    old = ev.MEMORY_LEAN
+    ev.MEMORY_LEAN = True
+    try:
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        o = TritonEvoformer(q, k, v, dev["mask"], bias)
+        o.backward(dev["dO"])
+        torch.cuda.synchronize()
+        peak = (torch.cuda.max_memory_allocated() - base) / 2 ** 20
+    finally:
+        ev.MEMORY_LEAN = old
+    print("C2 memory-lean peak %.2f MiB" % peak, flush=True)
+    assert peak <= 155.5
+
+
 def test_config5_peak_activation_memory():
     """C5 [1, 768, 768, 4, 32]: peak extra memory of fwd+bwd stays at the O(N*S*H*D) bound — O, dQ, dK,
     dV (144 MiB each) + LSE, delta, dBias (9 MiB each) — plus the declared workspace (the 9 MiB tiled copy of
