@@ -19,6 +19,7 @@
 #include "../../include/megafold_amd.h"
 #include "capi_common.h"
 #include "common.h"
+#include <type_traits>
 
 namespace mf {
 namespace {
@@ -344,10 +345,10 @@ __global__ void __launch_bounds__(256) opm_dw_reduce_kernel(const OpmDwParams p)
 //   unit        = (batch, block of 8 positions o, half of the 32 values f); its 128 x 128 result stays in registers
 //   job         = a unit and a tile of 4 positions t; a work-group walks over a contiguous run of jobs and writes one
 //                 partial piece per unit it touches (at most two); opm_dab_reduce_kernel adds the pieces of a unit
-//   stage A     wavefront w: dO rows (f_local = 2 w, 2 w + 1) x 32 h for the 32 pairs of the tile, wt resident in
-//               registers (A operand), dOut rows from LDS; laid into LDS as pair rows of 512 values
-//   stage B     wavefront (rt, sh): rows (2 positions o, 16 f) x 64 values s, contraction over (t, h) = 128:
-//               dO rows as plain fragments, the operand rows through transposing LDS reads
+//   stage A     wavefronts 0-3, wavefront w: dO rows (f_local = 4 w .. 4 w + 3) x 32 h for the 32 pairs of the tile, wt
+//               resident in registers (A operand), dOut rows from LDS; laid into LDS as pair rows of 512 values
+//   stage B     wavefronts 4-7, wavefront (rt2, sh): rows (4 positions o, 16 f) x 64 values s, contraction over
+//               (t, h) = 128: dO rows as plain fragments, the operand rows through transposing LDS reads
 // The tile's 128 operand rows and 32 dOut rows arrive by direct loads, double buffered, and so is the dO tile: between
 // two barriers the work-group runs stage B of job j and stage A of job j + 1, whose chains are independent (one
 // barrier per job, and each stage covers the LDS latencies of the other).
@@ -373,7 +374,6 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
   const int t512 = threadIdx.x;
   const int wv = __builtin_amdgcn_readfirstlane(t512 >> 6);
   const int l = t512 & 63, x = l & 31, g = l >> 5;
-  const int rt = wv & 3, sh = wv >> 2;
   const int n = p.n;
   const int j_begin = blockIdx.x * p.per_group;
   const int j_end = min(p.jobs, j_begin + p.per_group);
@@ -413,110 +413,143 @@ __global__ void __launch_bounds__(512, 1) opm_dab_kernel(const OpmDabParams p) {
     dma16((unsigned)(pair * 256 + ((pos ^ (r & 15)) << 4)), dbase, lds0 + DAB_LDS_D + buf * 8192 + wv * 1024);
   };
 
-  frag wf[2][8];
-  f32x16 acc[2] = {acc_zero(), acc_zero()};
-  int cur_unit = -1, cur_fh = -1, piece = 0;
-  auto flush = [&](int pc) {                       // register r of lane (x, g): row 8 (r >> 2) + 4 g + (r & 3), column x
-    float* dst = p.part + ((int64_t)blockIdx.x * 2 + pc) * 128 * 128;
+  // Roles: wavefronts 0-3 run stage A (wavefront w: four values f, wt resident), wavefronts 4-7 stage B (wavefront
+  // (rt2, sh2): 64 rows x 64 columns of the unit's result in registers).  Larger tiles per wavefront than with all
+  // eight on both stages: a third less LDS traffic, which bounds this kernel.  The two roles run separate loops with
+  // the same barriers and the same direct loads, so that each role's registers are only live in its own loop.
+  const int cw = wv & 3, rt2 = cw & 1, sh2 = cw >> 1;
+  auto run = [&](auto role) {
+    constexpr bool A = decltype(role)::value;      // true: stage A wavefront
+    frag wf[A ? 4 : 1][8];
+    f32x16 acc[2][2];
+    if constexpr (!A) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        dst[(rt * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + sh * 64 + c * 32 + x] = acc[c][r];
-  };
-  // rows f * 32 + h of wt for this wavefront's two values f, h permuted so that a register holds 16 g + r
-  auto load_wf = [&](int fh) {
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      const T* wrow = reinterpret_cast<const T*>(p.wt) + (int64_t)((fh * 16 + 2 * wv + a) * 32 + unperm32(x)) * 128 + 8 * g;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) wf[a][ks] = ld8<T>(wrow + 16 * ks);
+      for (int a = 0; a < 2; ++a) { acc[a][0] = acc_zero(); acc[a][1] = acc_zero(); }
     }
-    cur_fh = fh;
-  };
-  // stage A of a job: dO rows of the tile's 32 pairs into dO tile `ob`
-  auto stage_a = [&](int job, int db, int ob) {
-    int bb, o0, fh, t0;
-    decode(job, bb, o0, fh, t0);
-    if (fh != cur_fh) {
-      load_wf(fh);
-      wait_vm<0>();
-    }
-    const unsigned char* Dt = smem + DAB_LDS_D + db * 8192;
-    f32x16 o[2] = {acc_zero(), acc_zero()};
+    int cur_unit = -1, cur_fh = -1, piece = 0;
+    auto flush = [&](int pc) {                     // register r of lane (x, g): row 8 (r >> 2) + 4 g + (r & 3), column x
+      if constexpr (!A) {
+        float* dst = p.part + ((int64_t)blockIdx.x * 2 + pc) * 128 * 128;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const frag df = ld8<T>(reinterpret_cast<const T*>(Dt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
-      o[0] = mma(wf[0][ks], df, o[0]);             // rows = h (16 g + r in register r), columns = pairs
-      o[1] = mma(wf[1][ks], df, o[1]);
-    }
-    const bool live = t0 + (x & 3) < n;            // pairs past the edge contribute nothing
-    unsigned char* orow = smem + DAB_LDS_O + ob * 32 * DAB_OSTR + x * DAB_OSTR;
+        for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+          for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int q = 4 * (2 * wv + a) + 2 * g + u;            // 16-byte chunk (f_local * 32 + 16 g + 8 u) / 8
-        st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), live ? acc_half<T>(o[a], u) : frag_zero<T>());
+            for (int r = 0; r < 16; ++r)
+              dst[((2 * rt2 + a) * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * 128 + sh2 * 64 + c * 32 + x] = acc[a][c][r];
       }
-  };
-  // stage B of a job: its dO tile `ob` against its operand rows `pb`
-  auto stage_b = [&](int pb, int ob) {
-    const unsigned char* Pt = smem + DAB_LDS_P + pb * 32768;
-    const unsigned char* Ob = smem + DAB_LDS_O + ob * 32 * DAB_OSTR;
-    const int a4 = (l >> 2) & 3;
-    const int ol = 2 * rt + (x >> 4), fl = x & 15;
+    };
+    // stage A of a job: dO rows of the tile's 32 pairs into dO tile `ob`
+    auto stage_a = [&](int job, int db, int ob) {
+      if constexpr (A) {
+        int bb, o0, fh, t0;
+        decode(job, bb, o0, fh, t0);
+        if (fh != cur_fh) {                        // rows f * 32 + h of wt for this wavefront's four values f, h permuted
+          cur_fh = fh;                             // so that a register holds 16 g + r
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const int q = 4 * fl + 2 * (ks & 1) + g;
-      const frag of = ld8<T>(reinterpret_cast<const T*>(Ob + (ol * 4 + (ks >> 1)) * DAB_OSTR + ((q ^ ((q >> 4) & 3)) << 4)));
+          for (int a = 0; a < 4; ++a) {
+            const T* wrow = reinterpret_cast<const T*>(p.wt) + (int64_t)((fh * 16 + 4 * cw + a) * 32 + unperm32(x)) * 128 + 8 * g;
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const int col = sh * 64 + c * 32 + plain_chunk(l);
-        const int r0 = 16 * ks + 8 * g + a4, r1 = r0 + 4;
-        const unsigned char* p0 = Pt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
-        const unsigned char* p1 = Pt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        s16x8 v;
+            for (int ks = 0; ks < 8; ++ks) wf[a][ks] = ld8<T>(wrow + 16 * ks);
+          }
+          wait_vm<0>();
+        }
+        const unsigned char* Dt = smem + DAB_LDS_D + db * 8192;
+        frag df[8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
-        acc[c] = mma(of, __builtin_bit_cast(frag, v), acc[c]);   // rows = (o, f), columns = s
+        for (int ks = 0; ks < 8; ++ks) df[ks] = ld8<T>(reinterpret_cast<const T*>(Dt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
+        const bool live = t0 + (x & 3) < n;        // pairs past the edge contribute nothing
+        unsigned char* orow = smem + DAB_LDS_O + ob * 32 * DAB_OSTR + x * DAB_OSTR;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          f32x16 o[2] = {acc_zero(), acc_zero()};
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks) {
+            o[0] = mma(wf[2 * half][ks], df[ks], o[0]);        // rows = h (16 g + r in register r), columns = pairs
+            o[1] = mma(wf[2 * half + 1][ks], df[ks], o[1]);
+          }
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              const int q = 4 * (4 * cw + 2 * half + a) + 2 * g + u;   // 16-byte chunk (f_local * 32 + 16 g + 8 u) / 8
+              st8<T>(reinterpret_cast<T*>(orow + ((q ^ ((q >> 4) & 3)) << 4)), live ? acc_half<T>(o[a], u) : frag_zero<T>());
+            }
+        }
       }
-    }
-  };
+    };
+    // stage B of a job: its dO tile `ob` against its operand rows `pb`
+    auto stage_b = [&](int pb, int ob) {
+      if constexpr (!A) {
+        const unsigned char* Pt = smem + DAB_LDS_P + pb * 32768;
+        const unsigned char* Ob = smem + DAB_LDS_O + ob * 32 * DAB_OSTR;
+        const int a4 = (l >> 2) & 3;
+        const int fl = x & 15;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const int q = 4 * fl + 2 * (ks & 1) + g;
+          frag of[2];
+#pragma unroll
+          for (int a = 0; a < 2; ++a) {
+            const int ol = 2 * (2 * rt2 + a) + (x >> 4);
+            of[a] = ld8<T>(reinterpret_cast<const T*>(Ob + (ol * 4 + (ks >> 1)) * DAB_OSTR + ((q ^ ((q >> 4) & 3)) << 4)));
+          }
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            const int col = sh2 * 64 + c * 32 + plain_chunk(l);
+            const int r0 = 16 * ks + 8 * g + a4, r1 = r0 + 4;
+            const unsigned char* p0 = Pt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
+            const unsigned char* p1 = Pt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            s16x8 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+            const frag pf = __builtin_bit_cast(frag, v);
+            acc[0][c] = mma(of[0], pf, acc[0][c]);               // rows = (o, f), columns = s
+            acc[1][c] = mma(of[1], pf, acc[1][c]);
+          }
+        }
+      }
+    };
 
-  // prologue: the first job's tiles and the second job's dOut rows, then stage A of the first job
-  issue_d(j_begin, 0);
-  issue_p(j_begin, 0);
-  if (j_begin + 1 < j_end) issue_d(j_begin + 1, 1);
-  wait_vm<0>();
-  __builtin_amdgcn_s_waitcnt(0xC07F);
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  stage_a(j_begin, 0, 0);
-  for (int job = j_begin; job < j_end; ++job) {
-    const int k = (job - j_begin) & 1;
-    const int unit = job / p.tiles_t;
-    if (unit != cur_unit) {
-      if (cur_unit >= 0) {
-        flush(piece);
-        ++piece;
-        acc[0] = acc_zero(); acc[1] = acc_zero();
-      }
-      cur_unit = unit;
-    }
-    wait_vm<0>();                                  // operand rows of this job, dOut rows of the next have arrived
+    // prologue: the first job's tiles and the second job's dOut rows, then stage A of the first job
+    issue_d(j_begin, 0);
+    issue_p(j_begin, 0);
+    if (j_begin + 1 < j_end) issue_d(j_begin + 1, 1);
+    wait_vm<0>();
     __builtin_amdgcn_s_waitcnt(0xC07F);
-    __builtin_amdgcn_s_barrier();                  // ... for every wavefront, and this job's dO tile is complete; the
-    asm volatile("" ::: "memory");                 // buffers requested below were last read before this barrier
-    if (job + 1 < j_end) issue_p(job + 1, k ^ 1);
-    if (job + 2 < j_end) issue_d(job + 2, k);
-    if (job + 1 < j_end) stage_a(job + 1, k ^ 1, k ^ 1);
-    stage_b(k, k);
-  }
-  flush(piece);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    stage_a(j_begin, 0, 0);
+    for (int job = j_begin; job < j_end; ++job) {
+      const int k = (job - j_begin) & 1;
+      const int unit = job / p.tiles_t;
+      if (unit != cur_unit) {
+        if (cur_unit >= 0) {
+          flush(piece);
+          ++piece;
+          if constexpr (!A) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) { acc[a][0] = acc_zero(); acc[a][1] = acc_zero(); }
+          }
+        }
+        cur_unit = unit;
+      }
+      wait_vm<0>();                                // operand rows of this job, dOut rows of the next have arrived
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();                // ... for every wavefront, and this job's dO tile is complete; the
+      asm volatile("" ::: "memory");               // buffers requested below were last read before this barrier
+      if (job + 1 < j_end) issue_p(job + 1, k ^ 1);
+      if (job + 2 < j_end) issue_d(job + 2, k);
+      if (job + 1 < j_end) stage_a(job + 1, k ^ 1, k ^ 1);
+      stage_b(k, k);
+    }
+    flush(piece);
+  };
+  if (wv < 4) run(std::true_type{});
+  else run(std::false_type{});
 }
 
 // res[b][(o0 + R >> 4) * 32 + fh * 16 + (R & 15)][s] = sum of the unit's pieces, in the order of the work-groups
