@@ -178,10 +178,10 @@ __global__ void __launch_bounds__(512, 1) opm_fused_kernel(const OpmParams p) {
 // with the outer blocks recomputed tile by tile as in the forward, never stored.  The accumulators of all
 // 1024 x 128 products would fill a compute unit's register file, so a work-group owns a QUARTER of the products
 // (e in [8 q, 8 q + 8): 256 rows of dWt) and forms only those columns of the outer blocks:
-//   stage 1   wavefront w: the 32 x 32 tile  rows d  x  columns (4 positions j, 8 values e)  of row i0 + w over the
-//             MSA rows; laid into LDS as pair rows of 256 products (e_local * 32 + d)
-//   stage 2   wavefront (kt, ch): dWt_q[64 products, 64 channels] += O^T dOut over the 32 pairs of the tile, both
-//             operands through transposing LDS reads (rows = pairs)
+//   stage 1   wavefronts 0-3, wavefront w: the two 32 x 32 tiles  rows d  x  columns (4 positions j, 8 values e)  of rows
+//             i0 + 2 w and i0 + 2 w + 1 over the MSA rows; laid into LDS as pair rows of 256 products (e_local * 32 + d)
+//   stage 2   wavefronts 4-7, wavefront (kt2, ch): dWt_q[128 products, 64 channels] += O^T dOut over the 32 pairs of the
+//             tile, both operands through transposing LDS reads (rows = pairs)
 // A tile's operand rows of b (32 rows of 256 bytes) and its 32 rows of dOut arrive by direct loads, double
 // buffered.  Work-group (q, group) walks over a contiguous run of pair tiles and writes its sums to
 // part[group][q]; opm_dw_reduce_kernel adds the groups in a fixed order.
@@ -189,7 +189,7 @@ constexpr int DW_OSTR = 512 + 32;               // bytes between pair rows of th
 constexpr int DW_LDS_B = 0;                     // two tiles of 32 operand rows x 256 bytes
 constexpr int DW_LDS_D = 2 * 8192;              // two tiles of 32 dOut rows x 256 bytes
 constexpr int DW_LDS_O = 4 * 8192;
-constexpr int DW_LDS_BYTES = DW_LDS_O + 32 * DW_OSTR;
+constexpr int DW_LDS_BYTES = DW_LDS_O + 2 * 32 * DW_OSTR;   // two outer-block buffers
 
 struct OpmDwParams {
   int B, n, tiles_j, tiles, per_group, groups;
@@ -207,27 +207,28 @@ __global__ void __launch_bounds__(512, 1) opm_dw_kernel(const OpmDwParams p) {
   const int t512 = threadIdx.x;
   const int wv = __builtin_amdgcn_readfirstlane(t512 >> 6);
   const int l = t512 & 63, x = l & 31, g = l >> 5;
-  const int kt = wv & 3, ch = wv >> 2;
   const int n = p.n;
   const int q = blockIdx.x & 3, group = blockIdx.x >> 2;
   const int t_begin = group * p.per_group;
   const int t_end = min(p.tiles, t_begin + p.per_group);
-
-  f32x16 acc[2][2];
-#pragma unroll
-  for (int a = 0; a < 2; ++a) { acc[a][0] = acc_zero(); acc[a][1] = acc_zero(); }
+  if (t_begin >= t_end) return;
 
   const unsigned lds0 = (unsigned)(unsigned long)((__attribute__((address_space(3))) unsigned char*)smem);
   // one direct load per thread and operand: LDS row r = t512 >> 4 (0..31), 16-byte position pos = t512 & 15 holds
   // chunk pos ^ (r & 15) of the row.  b: row (j0 + (r >> 3)) * 32 + 8 q + (r & 7); dOut: pair (i0 + (r >> 2), j0 + (r & 3))
-  auto issue = [&](int tile, int buf) {
+  auto issue_b = [&](int tile, int buf) {
     const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
-    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+    const int j0 = (rem % p.tiles_j) * 4;
     const int r = t512 >> 4, pos = t512 & 15, chunk = (pos ^ (r & 15)) << 4;
     int j = j0 + (r >> 3);
     j = j < n ? j : n - 1;
     const char* bbase = reinterpret_cast<const char*>(p.b) + (int64_t)bb * n * 32 * 256;
     dma16((unsigned)((j * 32 + 8 * q + (r & 7)) * 256 + chunk), bbase, lds0 + DW_LDS_B + buf * 8192 + wv * 1024);
+  };
+  auto issue_d = [&](int tile, int buf) {
+    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+    const int r = t512 >> 4, pos = t512 & 15, chunk = (pos ^ (r & 15)) << 4;
     int i = i0 + (r >> 2), jd = j0 + (r & 3);
     i = i < n ? i : n - 1;
     jd = jd < n ? jd : n - 1;
@@ -235,85 +236,125 @@ __global__ void __launch_bounds__(512, 1) opm_dw_kernel(const OpmDwParams p) {
     dma16((unsigned)((i * n + jd) * 256 + chunk), dbase, lds0 + DW_LDS_D + buf * 8192 + wv * 1024);
   };
 
-  unsigned char* Ob = smem + DW_LDS_O;
-  frag af[8];
-  int cur_i0 = -1, cur_b = -1;
-  if (t_begin < t_end) issue(t_begin, 0);
-  for (int tile = t_begin; tile < t_end; ++tile) {
-    const int buf = (tile - t_begin) & 1;
-    const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
-    const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
-    if (i0 != cur_i0 || bb != cur_b) {             // rows d of position i0 + wv (columns of the block: permuted)
-      int i = i0 + wv;
-      i = i < n ? i : n - 1;
-      const T* arow = reinterpret_cast<const T*>(p.a) + ((int64_t)bb * n * 32 + i * 32 + unperm32(x)) * 128 + 8 * g;
+  // Roles: wavefronts 0-3 form the outer blocks (wavefront w: rows i0 + 2 w and i0 + 2 w + 1), wavefronts 4-7 contract
+  // them with dOut (wavefront (kt2, ch): 128 products x 64 channels in registers).  Between two barriers the second
+  // group works on tile t while the first prepares tile t + 1 in the other outer-block buffer.  Separate loops with the
+  // same barriers and direct loads, so that each role's registers are only live in its own loop.
+  const int cw = wv & 3, kt2 = cw & 1, ch = cw >> 1;
+  auto run = [&](auto role) {
+    constexpr bool A = decltype(role)::value;      // true: stage 1 wavefront
+    frag af[A ? 2 : 1][8];
+    f32x16 acc[4][2];
+    if constexpr (!A) {
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) af[ks] = ld8<T>(arow + 16 * ks);
-      cur_i0 = i0; cur_b = bb;
+      for (int a = 0; a < 4; ++a) { acc[a][0] = acc_zero(); acc[a][1] = acc_zero(); }
     }
-    wait_vm<0>();                                  // this tile's rows have arrived
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    __builtin_amdgcn_s_barrier();                  // ... for every wavefront; the other slots and the outer-block
-    asm volatile("" ::: "memory");                 // buffer are free (their readers are past the preceding tile)
-    if (tile + 1 < t_end) issue(tile + 1, buf ^ 1);
-    // ---- stage 1
-    {
-      const unsigned char* Bt = smem + DW_LDS_B + buf * 8192;
-      f32x16 o = acc_zero();
+    int cur_i0 = -1, cur_b = -1;
+    auto stage1 = [&](int tile, int bbuf, int ob) {
+      if constexpr (A) {
+        const int bb = tile / (p.tiles / p.B), rem = tile % (p.tiles / p.B);
+        const int i0 = (rem / p.tiles_j) * 8, j0 = (rem % p.tiles_j) * 4;
+        if (i0 != cur_i0 || bb != cur_b) {         // rows d of the two positions (columns of the blocks: permuted)
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const frag bf = ld8<T>(reinterpret_cast<const T*>(Bt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
-        o = mma(af[ks], bf, o);                    // rows = d (16 g + r in register r), columns = (j, e_local) = lane x
-      }
-      const int jj = x >> 3, el = x & 7;
-      const bool live = i0 + wv < n && j0 + jj < n;  // pairs past the edge contribute nothing
-      unsigned char* orow = Ob + (wv * 4 + jj) * DW_OSTR + (el * 32 + 16 * g) * 2;
-      st8<T>(reinterpret_cast<T*>(orow), live ? acc_half<T>(o, 0) : frag_zero<T>());
-      st8<T>(reinterpret_cast<T*>(orow + 16), live ? acc_half<T>(o, 1) : frag_zero<T>());
-    }
-    barrier_keep_vm<63>();                         // LDS hand-over only: the next tile keeps travelling
-    // ---- stage 2
-    {
-      const unsigned char* Dt = smem + DW_LDS_D + buf * 8192;
-      const int a4 = (l >> 2) & 3;
+          for (int u = 0; u < 2; ++u) {
+            int i = i0 + 2 * cw + u;
+            i = i < n ? i : n - 1;
+            const T* arow = reinterpret_cast<const T*>(p.a) + ((int64_t)bb * n * 32 + i * 32 + unperm32(x)) * 128 + 8 * g;
 #pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        frag of[2], df[2];
+            for (int ks = 0; ks < 8; ++ks) af[u][ks] = ld8<T>(arow + 16 * ks);
+          }
+          cur_i0 = i0; cur_b = bb;
+          wait_vm<0>();
+        }
+        const unsigned char* Bt = smem + DW_LDS_B + bbuf * 8192;
+        f32x16 o[2] = {acc_zero(), acc_zero()};
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const frag bf = ld8<T>(reinterpret_cast<const T*>(Bt + x * 256 + (((2 * ks + g) ^ (x & 15)) << 4)));
+          o[0] = mma(af[0][ks], bf, o[0]);         // rows = d (16 g + r in register r), columns = (j, e_local) = lane x
+          o[1] = mma(af[1][ks], bf, o[1]);
+        }
+        const int jj = x >> 3, el = x & 7;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          of[u] = TrRead<T>::read(reinterpret_cast<const T*>(Ob), DW_OSTR / 2, 16 * st, g, l,
-                                  kt * 64 + u * 32 + plain_chunk(l), kt * 64 + u * 32 + x);
-          // dOut rows are swizzled: the two 8-byte runs a lane points at lie in rows r0 and r0 + 4
-          const int col = ch * 64 + u * 32 + plain_chunk(l);                 // element column of the run
-          const int r0 = 16 * st + 8 * g + a4, r1 = r0 + 4;
-          const unsigned char* p0 = Dt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
-          const unsigned char* p1 = Dt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
-          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
-          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
-          typedef short s16x8 __attribute__((ext_vector_type(8)));
-          s16x8 v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
-          df[u] = __builtin_bit_cast(frag, v);
+          const int il = 2 * cw + u;
+          const bool live = i0 + il < n && j0 + jj < n;        // pairs past the edge contribute nothing
+          unsigned char* orow = smem + DW_LDS_O + ob * 32 * DW_OSTR + (il * 4 + jj) * DW_OSTR + (el * 32 + 16 * g) * 2;
+          st8<T>(reinterpret_cast<T*>(orow), live ? acc_half<T>(o[u], 0) : frag_zero<T>());
+          st8<T>(reinterpret_cast<T*>(orow + 16), live ? acc_half<T>(o[u], 1) : frag_zero<T>());
         }
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int c = 0; c < 2; ++c) acc[a][c] = mma(of[a], df[c], acc[a][c]);   // rows = products, columns = channels
       }
+    };
+    auto stage2 = [&](int dbuf, int ob) {
+      if constexpr (!A) {
+        const unsigned char* Dt = smem + DW_LDS_D + dbuf * 8192;
+        const T* Ob = reinterpret_cast<const T*>(smem + DW_LDS_O + ob * 32 * DW_OSTR);
+        const int a4 = (l >> 2) & 3;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          frag df[2];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            // dOut rows are swizzled: the two 8-byte runs a lane points at lie in rows r0 and r0 + 4
+            const int col = ch * 64 + u * 32 + plain_chunk(l);               // element column of the run
+            const int r0 = 16 * st + 8 * g + a4, r1 = r0 + 4;
+            const unsigned char* p0 = Dt + r0 * 256 + ((((col >> 3) ^ (r0 & 15)) << 4) | ((col & 4) << 1));
+            const unsigned char* p1 = Dt + r1 * 256 + ((((col >> 3) ^ (r1 & 15)) << 4) | ((col & 4) << 1));
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0));
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p1));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            s16x8 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[e + 4] = hi[e]; }
+            df[u] = __builtin_bit_cast(frag, v);
+          }
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const int k0 = kt2 * 128 + a * 32;
+            const frag of = TrRead<T>::read(Ob, DW_OSTR / 2, 16 * st, g, l, k0 + plain_chunk(l), k0 + x);
+            acc[a][0] = mma(of, df[0], acc[a][0]);               // rows = products, columns = channels
+            acc[a][1] = mma(of, df[1], acc[a][1]);
+          }
+        }
+      }
+    };
+
+    // prologue: operand rows of the first two tiles and dOut rows of the first, then the first tile's outer blocks
+    issue_b(t_begin, 0);
+    issue_d(t_begin, 0);
+    if (t_begin + 1 < t_end) issue_b(t_begin + 1, 1);
+    wait_vm<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    stage1(t_begin, 0, 0);
+    for (int tile = t_begin; tile < t_end; ++tile) {
+      const int k = (tile - t_begin) & 1;
+      wait_vm<0>();                                // dOut rows of this tile, operand rows of the next have arrived
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();                // ... for every wavefront, and this tile's outer blocks are complete;
+      asm volatile("" ::: "memory");               // the buffers requested below were last read before this barrier
+      if (tile + 2 < t_end) issue_b(tile + 2, k);
+      if (tile + 1 < t_end) issue_d(tile + 1, k ^ 1);
+      if (tile + 1 < t_end) stage1(tile + 1, k ^ 1, k ^ 1);
+      stage2(k, k);
     }
-  }
-  // ---- this work-group's sums: register r of lane (x, g) is row 8 (r >> 2) + 4 g + (r & 3), column x of its tile
-  float* dst = p.part + ((int64_t)group * 4 + q) * 256 * 128;
+    // ---- this work-group's sums: register r of lane (x, g) is row 8 (r >> 2) + 4 g + (r & 3), column x of its tile
+    if constexpr (!A) {
+      float* dst = p.part + ((int64_t)group * 4 + q) * 256 * 128;
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = kt * 64 + a * 32 + 8 * (r >> 2) + 4 * g + (r & 3), col = ch * 64 + c * 32 + x;
-        dst[row * 128 + col] = acc[a][c][r];
-      }
+          for (int r = 0; r < 16; ++r) {
+            const int row = kt2 * 128 + a * 32 + 8 * (r >> 2) + 4 * g + (r & 3), col = ch * 64 + c * 32 + x;
+            dst[row * 128 + col] = acc[a][c][r];
+          }
+    }
+  };
+  if (wv < 4) run(std::true_type{});
+  else run(std::false_type{});
 }
 
 // dwt[q * 256 + row][c] = sum over the groups, in their order
