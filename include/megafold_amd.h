@@ -324,6 +324,17 @@ int mf_pwa_softmax_bwd(const mf_pwa_args* a);
 int mf_opm_fused_fwd(const void* a, const void* b, const void* w, const void* bias, void* out, int32_t B, int32_t n,
                      int32_t dtype, void* stream);
 
+/* The two operands of mf_opm_fused_fwd from the hidden projection, and the way back for their gradients
+ * (megafold/model/megafold.py:788-807: MSA-row mask and the division by the number of rows as row_scale, the pair
+ * mask as a position mask on either side):
+ *   unpack = 0:  a[b, i*32 + d, s] = hidden[b, s, i, d] * row_scale[b, s] * pos[b, i]   (rounded once)
+ *                b[b, i*32 + e, s] = hidden[b, s, i, 32 + e] * pos[b, i];  columns S..127 are written as zero
+ *   unpack = 1:  hidden[b, s, i, d] = a[...] * row_scale[b, s] * pos[b, i],  hidden[b, s, i, 32 + e] = b[...] * pos[b, i]
+ *   hidden : [B, S, n, ldh >= 64] (ldh = element stride of a position); row_scale : [B, S] float;
+ *   pos : [B, n] bytes (0 = masked) or NULL; a, b : [B, n*32, 128]; S <= 128; 16-bit element types. */
+int mf_opm_pack(void* hidden, int64_t ldh, const float* row_scale, const void* pos, void* a, void* b, int32_t B, int32_t S,
+                int32_t n, int32_t unpack, int32_t dtype, void* stream);
+
 /* Gradient of that projection weight, the outer blocks formed again tile by tile and never stored
  * (autograd of megafold/model/megafold.py:807-812 with respect to to_pairwise_repr.weight):
  *   dwt[e*32 + d, c] = sum_{b,i,j} (sum_s a[b, i*32 + d, s] * b[b, j*32 + e, s]) * dout[b, i, j, c]

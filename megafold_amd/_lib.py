@@ -108,6 +108,8 @@ SYMBOLS = {
     "mf_opm_dab_workspace_bytes": (C.c_uint64, [C.c_int32, C.c_int32]),
     "mf_opm_dab": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32,
                              C.c_int32, C.c_int32, C.c_void_p]),
+    "mf_opm_pack": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                              C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "mf_opm_fused_fwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
                                    C.c_void_p]),
     "mf_pwa_softmax_fwd": (C.c_int, [C.POINTER(PwaArgs)]),

@@ -612,6 +612,83 @@ __global__ void __launch_bounds__(256) opm_dab_reduce_kernel(const OpmDabParams 
   dst[0] = (T)sum[0]; dst[1] = (T)sum[1]; dst[2] = (T)sum[2]; dst[3] = (T)sum[3];
 }
 
+
+// ================================================================================================
+// Operands of the kernels above from the hidden projection, and the way back for the gradients.
+//   pack    a[b, i*32 + d, s] = hidden[b, s, i, d] * row_scale[b, s] * pos[b, i]        (one rounding)
+//           b[b, i*32 + e, s] = hidden[b, s, i, 32 + e] * pos[b, i]                      s >= S: zero (128 columns)
+//   unpack  dhidden[b, s, i, d] = da[b, i*32 + d, s] * row_scale[b, s] * pos[b, i],  dhidden[b, s, i, 32 + e] = db[...] * pos
+// (megafold.py:788-807: the MSA-row mask and the division by the number of rows as row_scale, the pair mask as the
+// position mask on either side).  A work-group moves 8 positions x 32 MSA rows through an LDS tile.
+struct OpmPackParams {
+  int B, S, n, unpack;
+  void* hidden; int64_t ldh;          // [B, S, n, ldh >= 64] (element stride of a position)
+  const float* row_scale;             // [B, S]
+  const unsigned char* pos;           // [B, n] or nullptr
+  void* a; void* b;                   // [B, n * 32, 128]
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) opm_pack_kernel(const OpmPackParams p) {
+  __shared__ T tile[8 * 64][32 + 2];                          // [(i_local, channel)][s_local]
+  const int t = threadIdx.x;
+  const int s0 = blockIdx.x * 32, i0 = blockIdx.y * 8, bb = blockIdx.z;
+  T* H = reinterpret_cast<T*>(p.hidden);
+  T* Aop = reinterpret_cast<T*>(p.a);
+  T* Bop = reinterpret_cast<T*>(p.b);
+  if (!p.unpack) {
+    // in: 8 threads per (s, i) row of 64 channels
+    for (int item = t; item < 32 * 8 * 8; item += 256) {
+      const int ch = item & 7, i_l = (item >> 3) & 7, s_l = item >> 6;
+      const int sidx = s0 + s_l, i = i0 + i_l;
+      frag_t<T> v = frag_zero<T>();
+      float f = 0.0f;
+      if (sidx < p.S && i < p.n) {
+        v = ld8<T>(H + (((int64_t)bb * p.S + sidx) * p.n + i) * p.ldh + 8 * ch);
+        f = p.pos ? (p.pos[(int64_t)bb * p.n + i] ? 1.0f : 0.0f) : 1.0f;
+        if (ch < 4) f *= p.row_scale[(int64_t)bb * p.S + sidx];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[i_l * 64 + 8 * ch + e][s_l] = (T)((float)v[e] * f);
+    }
+    __syncthreads();
+    // out: 4 threads per operand row (32 MSA rows = 64 bytes)
+    for (int item = t; item < 8 * 64 * 4; item += 256) {
+      const int c4 = item & 3, row = item >> 2, i_l = row >> 6, c = row & 63;
+      const int i = i0 + i_l;
+      if (i < p.n) {
+        frag_t<T> v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = tile[row][8 * c4 + e];
+        T* dst = (c < 32 ? Aop : Bop) + (((int64_t)bb * p.n + i) * 32 + (c & 31)) * 128 + s0 + 8 * c4;
+        st8<T>(dst, v);
+      }
+    }
+  } else {
+    for (int item = t; item < 8 * 64 * 4; item += 256) {
+      const int c4 = item & 3, row = item >> 2, i_l = row >> 6, c = row & 63;
+      const int i = i0 + i_l;
+      frag_t<T> v = frag_zero<T>();
+      if (i < p.n) v = ld8<T>((c < 32 ? Aop : Bop) + (((int64_t)bb * p.n + i) * 32 + (c & 31)) * 128 + s0 + 8 * c4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[row][8 * c4 + e] = v[e];
+    }
+    __syncthreads();
+    for (int item = t; item < 32 * 8 * 8; item += 256) {
+      const int ch = item & 7, i_l = (item >> 3) & 7, s_l = item >> 6;
+      const int sidx = s0 + s_l, i = i0 + i_l;
+      if (sidx < p.S && i < p.n) {
+        float f = p.pos ? (p.pos[(int64_t)bb * p.n + i] ? 1.0f : 0.0f) : 1.0f;
+        if (ch < 4) f *= p.row_scale[(int64_t)bb * p.S + sidx];
+        frag_t<T> v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (T)((float)tile[i_l * 64 + 8 * ch + e][s_l] * f);
+        st8<T>(H + (((int64_t)bb * p.S + sidx) * p.n + i) * p.ldh + 8 * ch, v);
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace mf
 
@@ -745,4 +822,24 @@ extern "C" int mf_opm_dab(const void* dout, const void* wt, const void* opnd, vo
   };
   return (int)(dtype == MF_DTYPE_BF16 ? launch(opm_dab_kernel<bf16_t>, opm_dab_reduce_kernel<bf16_t>)
                                       : launch(opm_dab_kernel<f16_t>, opm_dab_reduce_kernel<f16_t>));
+}
+
+extern "C" int mf_opm_pack(void* hidden, int64_t ldh, const float* row_scale, const void* pos, void* a, void* b, int32_t B,
+                           int32_t S, int32_t n, int32_t unpack, int32_t dtype, void* stream) {
+  clear_error();
+  if (!hidden || !row_scale || !a || !b) return fail(MF_ERR_NULL, "hidden, row_scale, a or b is NULL");
+  if (!aligned16(hidden) || !aligned16(a) || !aligned16(b)) return fail(MF_ERR_ALIGN, "operands must be 16-byte aligned");
+  if (B <= 0 || n <= 0 || S <= 0 || S > 128) return fail(MF_ERR_SHAPE, "need B, n > 0 and 0 < S <= 128 (got %d, %d, %d)", B, n, S);
+  if (ldh < 64 || ldh % 8 != 0) return fail(MF_ERR_STRIDE, "ldh=%lld: need a multiple of 8, at least 64", (long long)ldh);
+  if (dtype != MF_DTYPE_F16 && dtype != MF_DTYPE_BF16) return fail(MF_ERR_DTYPE, "dtype %d unsupported: f16 / bf16", dtype);
+  if (B > 65535 || (n + 7) / 8 > 65535) return fail(MF_ERR_SHAPE, "dimensions exceed the launch grid");
+  OpmPackParams p{};
+  p.B = B; p.S = S; p.n = n; p.unpack = unpack ? 1 : 0;
+  p.hidden = hidden; p.ldh = ldh; p.row_scale = row_scale; p.pos = static_cast<const unsigned char*>(pos); p.a = a; p.b = b;
+  // pack writes all 128 columns of the operands (zeros past S); unpack only reads the first S
+  const dim3 grid((unsigned)(unpack ? (S + 31) / 32 : 4), (unsigned)((n + 7) / 8), (unsigned)B);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == MF_DTYPE_BF16) hipLaunchKernelGGL(opm_pack_kernel<bf16_t>, grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(opm_pack_kernel<f16_t>, grid, dim3(256), 0, st, p);
+  return (int)hipGetLastError();
 }

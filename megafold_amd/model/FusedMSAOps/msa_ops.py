@@ -41,7 +41,7 @@ from ..FusedTriangleAttention.triangle_attention import sigmoid_gate_backward
 from ..gate import sigmoid_gate
 from ..linear import linear_no_bias
 
-__all__ = ["MSAPairWeightedAveraging", "OuterProductMean", "PairWeightedAverageFunction", "OuterProductProjectFunction"]
+__all__ = ["MSAPairWeightedAveraging", "OuterProductMean", "PairWeightedAverageFunction", "OuterProductMeanFunction"]
 
 
 def _pwa_args(b, s, n, h, d, dtype, device):
@@ -203,16 +203,21 @@ class OuterProductMean(nn.Module):
     def forward(self, msa: torch.Tensor, *, mask: Optional[torch.Tensor] = None,
                 msa_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         b, s, n, _ = msa.shape
-        a, b_ = self.to_hidden(msa).chunk(2, dim=-1)                             # [b, s, n, dh] each (views)
-        dtype, dh = a.dtype, a.shape[-1]
+        hidden = self.to_hidden(msa)                                             # [b, s, n, 2 dh]
+        dtype, dh = hidden.dtype, hidden.shape[-1] // 2
+        lin = self.to_pairwise_repr
         # Everything elementwise is applied to the two small operands instead of the [b, n, n, dh*dh] product:
         # the MSA-row mask (0/1, so masking one operand equals masking both), the division by the number of kept
         # rows, and the pair mask mask_i * mask_j as a row mask on each side.
         if msa_mask is not None:
             inv = 1.0 / msa_mask.to(torch.float32).sum(-1).clamp(min=self.eps)               # [b]
-            fa = (msa_mask.to(torch.float32) * inv[:, None])[:, :, None, None]
+            row_scale = msa_mask.to(torch.float32) * inv[:, None]                            # [b, s]
         else:
-            fa = torch.full((1, 1, 1, 1), 1.0 / s, dtype=torch.float32, device=msa.device)
+            row_scale = torch.full((b, s), 1.0 / s, dtype=torch.float32, device=msa.device)
+        if (dh == 32 and lin.out_features == 128 and s <= 128 and dtype in (torch.float16, torch.bfloat16) and hidden.is_cuda):
+            return OuterProductMeanFunction.apply(hidden, row_scale, mask, lin.weight, lin.bias)
+        a, b_ = hidden.chunk(2, dim=-1)                                          # [b, s, n, dh] each (views)
+        fa = row_scale[:, :, None, None]
         fb = None
         if mask is not None:
             pos = mask.to(torch.float32)[:, None, :, None]                                   # [b, 1, n, 1]
@@ -223,9 +228,6 @@ class OuterProductMean(nn.Module):
         # operand matrices [(i d), s] with the contraction axis contiguous
         A = a.permute(0, 2, 3, 1).reshape(b, n * dh, s)
         B = b_.permute(0, 2, 3, 1).reshape(b, n * dh, s)
-        lin = self.to_pairwise_repr
-        if (dh == 32 and lin.out_features == 128 and s <= 128 and dtype in (torch.float16, torch.bfloat16) and A.is_cuda):
-            return OuterProductProjectFunction.apply(A, B, lin.weight, lin.bias, n)
         return _outer_project_reference(A, B, lin.weight, lin.bias, n, dh)
 
 
@@ -239,65 +241,68 @@ def _outer_project_reference(A, B, weight, bias, n, dh):
     return out + bias.to(out.dtype) if bias is not None else out
 
 
-class OuterProductProjectFunction(torch.autograd.Function):
-    """``out[b, i, j, :] = W . (sum_s A[b, (i d), s] B[b, (j e), s])_(d e) + bias`` through ``mf_opm_fused_fwd``: the
-    ``[n, n, dh * dh]`` outer product never exists, in the forward or in the backward (``mf_opm_dw`` for the weight,
-    ``mf_opm_dab`` for each operand: the outer blocks and their gradient are formed tile by tile in LDS)."""
+class OuterProductMeanFunction(torch.autograd.Function):
+    """``out[b, i, j, :] = W . (sum_s a[b, s, i, :] (x) b[b, s, j, :])_(d e) + bias`` with ``a | b`` the two halves of
+    ``hidden`` scaled by ``row_scale[b, s]`` (first half only) and the position mask: operands packed by ``mf_opm_pack``,
+    outer blocks and projection in one kernel (``mf_opm_fused_fwd``).  The ``[n, n, dh * dh]`` outer product never
+    exists, in the forward or in the backward (``mf_opm_dw`` for the weight, ``mf_opm_dab`` for each operand: the outer
+    blocks and their gradient are formed tile by tile in LDS; ``mf_opm_pack`` again for the way back to ``hidden``)."""
 
     @staticmethod
-    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
-    def forward(ctx, A, B, weight, bias, n):
-        b, rows, s = A.shape
-        dtype = A.dtype
-        with torch.cuda.device(A.device):
-            # zero padded to 128 columns; the weight with its two hidden indices exchanged (column e * 32 + d)
-            Ap = torch.zeros((b, rows, 128), dtype=dtype, device=A.device)
-            Bp = torch.zeros((b, rows, 128), dtype=dtype, device=A.device)
-            Ap[:, :, :s] = A
-            Bp[:, :, :s] = B
+    def forward(ctx, hidden, row_scale, mask, weight, bias):
+        b, s, n, _ = hidden.shape
+        dtype, dev = hidden.dtype, hidden.device
+        hidden = hidden if hidden.is_contiguous() else hidden.contiguous()
+        lib = _lib.lib()
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            pos = mask.to(torch.uint8).contiguous() if mask is not None else None
+            row_scale = row_scale.to(torch.float32).contiguous()
+            Ap = torch.empty((b, n * 32, 128), dtype=dtype, device=dev)
+            Bp = torch.empty((b, n * 32, 128), dtype=dtype, device=dev)
+            _lib.check(lib.mf_opm_pack(hidden.data_ptr(), hidden.shape[-1], row_scale.data_ptr(),
+                                       pos.data_ptr() if pos is not None else None, Ap.data_ptr(), Bp.data_ptr(),
+                                       b, s, n, 0, _lib.dtype_code(dtype), stream), "mf_opm_pack")
+            # the weight with its two hidden indices exchanged (column e * 32 + d)
             wp = weight.to(dtype).view(128, 32, 32).transpose(1, 2).contiguous()
-            out = torch.empty((b, n, n, 128), dtype=dtype, device=A.device)
-            _lib.check(_lib.lib().mf_opm_fused_fwd(Ap.data_ptr(), Bp.data_ptr(), wp.data_ptr(),
-                                                   bias.to(dtype).data_ptr() if bias is not None else None,
-                                                   out.data_ptr(), b, n, _lib.dtype_code(dtype),
-                                                   torch.cuda.current_stream(A.device).cuda_stream),
-                       "mf_opm_fused_fwd")
-        ctx.save_for_backward(Ap, Bp, weight, bias)
-        ctx.n, ctx.s = n, s
+            out = torch.empty((b, n, n, 128), dtype=dtype, device=dev)
+            _lib.check(lib.mf_opm_fused_fwd(Ap.data_ptr(), Bp.data_ptr(), wp.data_ptr(),
+                                            bias.to(dtype).data_ptr() if bias is not None else None,
+                                            out.data_ptr(), b, n, _lib.dtype_code(dtype), stream), "mf_opm_fused_fwd")
+        ctx.save_for_backward(Ap, Bp, weight, bias, row_scale, pos)
+        ctx.dims = (b, s, n, hidden.shape[-1])
         return out
 
     @staticmethod
-    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dout):
-        Ap, Bp, weight, bias = ctx.saved_tensors
-        b, rows, _ = Ap.shape
-        n, dh, s = ctx.n, 32, ctx.s
-        A, B = Ap[:, :, :s], Bp[:, :, :s]
-        dout2 = dout.reshape(b * n * n, 128).to(Ap.dtype).contiguous()
-        w = weight.to(Ap.dtype)
-        # weight gradient: the outer blocks are formed again tile by tile inside mf_opm_dw, never stored;
-        # the kernel returns [e * 32 + d, channel] in fp32
+        Ap, Bp, weight, bias, row_scale, pos = ctx.saved_tensors
+        b, s, n, width = ctx.dims
+        dh, dtype, dev = 32, Ap.dtype, Ap.device
+        dout2 = dout.reshape(b * n * n, 128).to(dtype).contiguous()
+        w = weight.to(dtype)
         lib = _lib.lib()
-        with torch.cuda.device(Ap.device):
-            nbytes = lib.mf_opm_dw_workspace_bytes(b, n)
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=Ap.device)
-            dwt = torch.empty((dh * dh, 128), dtype=torch.float32, device=Ap.device)
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            code = _lib.dtype_code(dtype)
+            # weight gradient: the outer blocks are formed again tile by tile inside mf_opm_dw, never stored;
+            # the kernel returns [e * 32 + d, channel] in fp32
+            nbytes = max(lib.mf_opm_dw_workspace_bytes(b, n), lib.mf_opm_dab_workspace_bytes(b, n))
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            dwt = torch.empty((dh * dh, 128), dtype=torch.float32, device=dev)
             _lib.check(lib.mf_opm_dw(Ap.data_ptr(), Bp.data_ptr(), dout2.data_ptr(), dwt.data_ptr(), ws.data_ptr(), nbytes,
-                                     b, n, _lib.dtype_code(Ap.dtype), torch.cuda.current_stream(Ap.device).cuda_stream),
-                       "mf_opm_dw")
-        dW = dwt.view(dh, dh, 128).permute(2, 1, 0).reshape(128, dh * dh)          # [channel, d * 32 + e]
-        dbias = dout2.sum(0, dtype=torch.float32).to(bias.dtype) if bias is not None else None
-        # operand gradients: tiles of dOut . W^T live in LDS between two products inside mf_opm_dab (once per side)
-        with torch.cuda.device(Ap.device):
+                                     b, n, code, stream), "mf_opm_dw")
+            # operand gradients: tiles of dOut . W^T live in LDS between two products inside mf_opm_dab (once per side)
             wt_a = w.t().contiguous()                                                        # row d * 32 + e
             wt_b = w.view(128, dh, dh).permute(2, 1, 0).reshape(dh * dh, 128).contiguous()   # row e * 32 + d
-            nbytes = lib.mf_opm_dab_workspace_bytes(b, n)
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=Ap.device)
             dAp, dBp = torch.empty_like(Ap), torch.empty_like(Bp)
-            stream = torch.cuda.current_stream(Ap.device).cuda_stream
             _lib.check(lib.mf_opm_dab(dout2.data_ptr(), wt_a.data_ptr(), Bp.data_ptr(), dAp.data_ptr(), ws.data_ptr(), nbytes,
-                                      b, n, 0, _lib.dtype_code(Ap.dtype), stream), "mf_opm_dab")
+                                      b, n, 0, code, stream), "mf_opm_dab")
             _lib.check(lib.mf_opm_dab(dout2.data_ptr(), wt_b.data_ptr(), Ap.data_ptr(), dBp.data_ptr(), ws.data_ptr(), nbytes,
-                                      b, n, 1, _lib.dtype_code(Ap.dtype), stream), "mf_opm_dab")
-        dA, dB = dAp[:, :, :s], dBp[:, :, :s]
-        return dA, dB, dW.to(weight.dtype), dbias, None
+                                      b, n, 1, code, stream), "mf_opm_dab")
+            dhidden = torch.empty((b, s, n, width), dtype=dtype, device=dev)
+            _lib.check(lib.mf_opm_pack(dhidden.data_ptr(), width, row_scale.data_ptr(),
+                                       pos.data_ptr() if pos is not None else None, dAp.data_ptr(), dBp.data_ptr(),
+                                       b, s, n, 1, code, stream), "mf_opm_pack")
+        dW = dwt.view(dh, dh, 128).permute(2, 1, 0).reshape(128, dh * dh)          # [channel, d * 32 + e]
+        dbias = dout2.sum(0, dtype=torch.float32).to(bias.dtype) if bias is not None else None
+        return dhidden, None, None, dW.to(weight.dtype), dbias

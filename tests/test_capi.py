@@ -360,6 +360,12 @@ def test_outer_product_mean_argument_errors():
     assert lib.mf_opm_dab(D, W, Bm, O, WS + 2, need, 2, 37, 0, bf16, None) == -5
     assert lib.mf_opm_dab(D, W, Bm, O, WS, need - 1, 2, 37, 1, bf16, None) == -6
     assert lib.mf_opm_dab(D, W, Bm, O, WS, need, 2, 37, 1, 7, None) == -3
+    RS = 0x70000
+    assert lib.mf_opm_pack(None, 64, RS, None, A, Bm, 1, 12, 16, 0, bf16, None) == -1
+    assert lib.mf_opm_pack(D, 64, RS, None, A + 8, Bm, 1, 12, 16, 0, bf16, None) == -5
+    assert lib.mf_opm_pack(D, 64, RS, None, A, Bm, 1, 129, 16, 0, bf16, None) == -2 and "S <= 128" in lib.mf_last_error().decode()
+    assert lib.mf_opm_pack(D, 60, RS, None, A, Bm, 1, 12, 16, 1, bf16, None) == -4
+    assert lib.mf_opm_pack(D, 64, RS, None, A, Bm, 1, 12, 16, 1, _lib.MF_F32, None) == -3
 
 
 def test_pair_weighted_averaging_argument_errors():
