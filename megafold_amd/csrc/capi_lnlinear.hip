@@ -144,8 +144,12 @@ extern "C" int mf_lnlinear_bwd(const mf_lnlinear_args* a) {
   const LnPlan pl = make_plan(a, true);
   const LnParams p = fill(a, pl, true);
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
-  hipError_t e = launch_ln_prep(p, false, stream);
-  if (e != hipSuccess) return (int)e;
+  hipError_t e = hipSuccess;
+  // the register-resident dx kernel forms its slice of gamma (.) W itself; every other path reads the prepared copies
+  if (!(a->act == MF_ACT_NONE && ln_bwd_takes_dx_add(a->dtype, a->K, a->N))) {
+    e = launch_ln_prep(p, false, stream);
+    if (e != hipSuccess) return (int)e;
+  }
   const void* dY = a->dout;
   if (a->act == MF_ACT_SWIGLU) {
     // recompute the pre-activation tile by tile and turn dh into dU = [da, dg]; where the shape allows it one pass

@@ -632,7 +632,8 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int kt = w & 3, nh = w >> 2;
   const int N = p.N, K = p.K;
-  const T* Wg = reinterpret_cast<const T*>(p.Wg);
+  const T* Wraw = reinterpret_cast<const T*>(p.W);
+  const T* gam = reinterpret_cast<const T*>(p.gamma);
   const T* X = reinterpret_cast<const T*>(p.x);
   T* dX = reinterpret_cast<T*>(p.dx);
   const T* DR = ADD ? reinterpret_cast<const T*>(p.dx_add) : nullptr;
@@ -648,7 +649,12 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
       const int r = item / YCH, c = item % YCH;
       const int k = 32 * ww + r;
       const bool ok = k < K && 8 * c < N;
-      tmp[i] = ld8<T>(Wg + (int64_t)(ok ? k : 0) * N + (ok ? 8 * c : 0));
+      // W' = gamma (.) W formed here, once per work-group, with the rounding of the preparation kernel: the
+      // backward of the plain linear form then needs no preparation launch at all
+      const frag wv = ld8<T>(Wraw + (int64_t)(ok ? k : 0) * N + (ok ? 8 * c : 0));
+      const float gk = to_f(gam[ok ? k : 0]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tmp[i][e] = (T)(gk * to_f(wv[e]));
     }
 #pragma unroll
     for (int i = 0; i < YPF; ++i) {
