@@ -30,7 +30,9 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
   using frag = frag_t<T>;
   constexpr int KS = KP / 16, CPR = KP / 8, KT = KP / 32;
   constexpr int RB = 32;
-  constexpr int WLDS = KP > 64 ? 16 : 8;            // PARTS: W' fragments per consumer kept in LDS
+  // normalised rows are read with transposing reads (four consecutive rows per 16 lanes): rows 8 banks apart
+  constexpr int XHSTR = (L::XSTR * (int)sizeof(T) / 4) % 64 == 4 ? L::XSTR + 8 : L::XSTR;
+  constexpr int WLDS = KP > 64 ? 15 : 8;            // PARTS: W' fragments per consumer kept in LDS
   constexpr int OSTR = 32 + 8;                      // row stride of a 32-column tile (elements)
   constexpr int TILE = 32 * OSTR;                   // one da or dg tile
   constexpr int PSET = 4 * TILE + 32;               // tiles of one producer: [2 buffers][da, dg], then 64 bytes that
@@ -38,8 +40,8 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T* Xs = reinterpret_cast<T*>(smem_raw);                          // [2][RB][XSTR]  raw rows
-  T* Xh = Xs + 2 * RB * L::XSTR;                                   // [3][RB][XSTR]  normalised rows
-  float* meanL = reinterpret_cast<float*>(Xh + 3 * RB * L::XSTR);  // [2][RB]
+  T* Xh = Xs + 2 * RB * L::XSTR;                                   // [3][RB][XHSTR]  normalised rows
+  float* meanL = reinterpret_cast<float*>(Xh + 3 * RB * XHSTR);    // [2][RB]
   float* rstdL = meanL + 2 * RB;                                   // [2][RB]
   float* csL = rstdL + 2 * RB;                                     // [4 * 2 * 32]
   float* bpL = csL + 4 * 2 * 32;
@@ -116,7 +118,7 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
       float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (to_f(xv[e]) - xmu) * rl;
-      st8<T>(Xh + (hbuf * RB + srow) * L::XSTR + 8 * sdc, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
+      st8<T>(Xh + (hbuf * RB + srow) * XHSTR + 8 * sdc, cvt8<T>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]));
     }
   };
 
@@ -262,7 +264,7 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
 #pragma unroll
           for (int b = 0; b < 2; ++b) bf[st][b] = TrRead<T>::read(tiles + b * TILE, OSTR, 16 * st, g, l, plain_chunk(l), x);
         }
-        if (a < KT) xf[slot] = TrRead<T>::read(xh, L::XSTR, 16 * st, g, l, 32 * a + plain_chunk(l), 32 * a + x);
+        if (a < KT) xf[slot] = TrRead<T>::read(xh, XHSTR, 16 * st, g, l, 32 * a + plain_chunk(l), 32 * a + x);
         if constexpr (PARTS) {
           if (dyw) {
 #pragma unroll
@@ -318,13 +320,13 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
       if (rb + 2 * Gx < nrb) fetch(rb + 2 * Gx);
       if (it > 0) {
         if constexpr (!PARTS) flush(rb - Gx, buf ^ 1);
-        consume(rb - Gx, buf ^ 1, Xh + ((it - 1) % 3) * RB * L::XSTR);
+        consume(rb - Gx, buf ^ 1, Xh + ((it - 1) % 3) * RB * XHSTR);
       }
     }
     barrier_keep_vm<63>();
     if (it > 0) {
       if constexpr (!PARTS) flush(rb - Gx, (it - 1) & 1);
-      consume(rb - Gx, (it - 1) & 1, Xh + ((it - 1) % 3) * RB * L::XSTR);
+      consume(rb - Gx, (it - 1) & 1, Xh + ((it - 1) % 3) * RB * XHSTR);
     }
 
     // ---- partial sums of this work-group: range blockIdx.x --------------------------------------------------
@@ -408,8 +410,9 @@ template <typename T> static bool swiglu_bwd_fused_ok(const LnParams& p) {
 template <typename T, int KP, bool PARTS> static hipError_t launch_swiglu_bwd_fused_k(const LnParams& p, hipStream_t stream) {
   using L = LnLayout<T, KP>;
   const int gy = (p.N / 2) / 128;
-  const size_t smem = (size_t)5 * 32 * L::XSTR * sizeof(T) + (size_t)4 * 32 * 4 + (size_t)2 * 4 * 2 * 32 * 4 +
-                      (size_t)((4 * 2 * 2 + 4) * 32 * 40 + 4 * 32) * sizeof(T) + (PARTS ? (size_t)4 * (KP > 64 ? 16 : 8) * 64 * 16 : 0);
+  constexpr int XHSTR = (L::XSTR * (int)sizeof(T) / 4) % 64 == 4 ? L::XSTR + 8 : L::XSTR;      // as in the kernel
+  const size_t smem = (size_t)32 * (2 * L::XSTR + 3 * XHSTR) * sizeof(T) + (size_t)4 * 32 * 4 + (size_t)2 * 4 * 2 * 32 * 4 +
+                      (size_t)((4 * 2 * 2 + 4) * 32 * 40 + 4 * 32) * sizeof(T) + (PARTS ? (size_t)4 * (KP > 64 ? 15 : 8) * 64 * 16 : 0);
   const size_t wst = (size_t)128 * L::XSTR * sizeof(T);           // weight staging aliases the tiles
   static_assert(sizeof(T) == 2, "");
   if (wst > (size_t)(4 * 2 * 2 + 4) * 32 * 40 * sizeof(T)) return hipErrorInvalidValue;
