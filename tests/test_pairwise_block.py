@@ -160,3 +160,73 @@ def test_fp32_residual_stream_under_autocast_stays_fp32(kind):
                 y2 = call(x2, False)
             y2.float().square().mean().backward()
             assert torch.equal(y, y2) and torch.equal(xg.grad, x2.grad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["pairwise_block", "attention_pair_bias", "msa_pair_weighted_averaging",
+                                  "outer_product_mean"])
+def test_blocks_replay_from_a_captured_graph(kind):
+    """Forward and backward of a block captured into HIP graphs (torch.cuda.make_graphed_callables) and replayed:
+    the library launches on the stream it is handed and neither allocates, clears memory with a memset node nor
+    synchronises, so a capture holds kernels only.  Every replay, with eager work of the same module and
+    synchronisations between the replays and with new input values each time, must reproduce the eager output, input
+    gradients and parameter gradients bit for bit."""
+    from megafold_amd.model.FusedAttentionPairBias import AttentionPairBias
+    from megafold_amd.model.FusedMSAOps import MSAPairWeightedAveraging, OuterProductMean
+    n, s = 72, 20
+    g = torch.Generator().manual_seed(17)
+    rnd = lambda *sh: torch.randn(*sh, generator=g).to(torch.bfloat16).cuda()
+    mask = torch.ones(1, n, dtype=torch.bool, device="cuda")
+    mask[:, n - 5:] = False
+
+    class Wrapped(torch.nn.Module):          # graphed callables take tensors only: the mask rides along as a constant
+        def __init__(self, inner, call):
+            super().__init__()
+            self.inner, self.call = inner, call
+
+        def forward(self, *tensors):
+            return self.call(self.inner, *tensors)
+
+    if kind == "pairwise_block":
+        mod = Wrapped(PairwiseBlock(dropout_row_prob=0.0, dropout_col_prob=0.0),
+                      lambda m, pair: m(pairwise_repr=pair, mask=mask))
+        shapes, oshape = [(1, n, n, 128)], (1, n, n, 128)
+    elif kind == "attention_pair_bias":
+        mod = Wrapped(AttentionPairBias(heads=16, dim_pairwise=128, dim=384, dim_head=64),
+                      lambda m, single, pair: m(single, pairwise_repr=pair, mask=mask))
+        shapes, oshape = [(1, n, 384), (1, n, n, 128)], (1, n, 384)
+    elif kind == "msa_pair_weighted_averaging":
+        mod = Wrapped(MSAPairWeightedAveraging(dim_msa=64, dim_pairwise=128, dim_head=32, heads=8),
+                      lambda m, msa, pair: m(msa=msa, pairwise_repr=pair, mask=mask))
+        shapes, oshape = [(1, s, n, 64), (1, n, n, 128)], (1, s, n, 64)
+    else:
+        mod = Wrapped(OuterProductMean(dim_msa=64, dim_pairwise=128, dim_hidden=32), lambda m, msa: m(msa, mask=mask))
+        shapes, oshape = [(1, s, n, 64)], (1, n, n, 128)
+    mod = mod.cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        for p in mod.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(p.dtype))
+
+    def fresh():
+        return tuple(rnd(*sh).requires_grad_() for sh in shapes)
+
+    def run(fn, args, dout):
+        out = fn(*args)
+        out.backward(dout)
+        res = [out.detach().clone()] + [a.grad.clone() for a in args] + [p.grad.clone() for p in mod.parameters()]
+        for t in list(args) + list(mod.parameters()):
+            t.grad = None
+        return res
+
+    cases = [(fresh(), rnd(*oshape)) for _ in range(3)]
+    want = [run(mod, a, d) for a, d in cases]
+    graphed = torch.cuda.make_graphed_callables(mod, fresh(), num_warmup_iters=3)
+    for rep in range(3):
+        for i, (a, d) in enumerate(cases):
+            got = run(graphed, a, d)
+            torch.cuda.synchronize()
+            for j, (x, y) in enumerate(zip(got, want[i])):
+                assert torch.equal(x, y), "replay %d, inputs %d, tensor %d differs from the eager result" % (rep, i, j)
+        eager = run(mod, *cases[rep])                        # the program's own eager work between the replays
+        torch.cuda.synchronize()
+        assert all(torch.equal(x, y) for x, y in zip(eager, want[rep]))
