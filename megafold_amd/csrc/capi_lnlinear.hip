@@ -16,7 +16,7 @@ namespace {
 struct LnPlan {
   int KP, R;
   int64_t rows_per_range;
-  uint64_t off_wt, off_cs, off_bp, off_wg, off_g, off_s, off_du, total;
+  uint64_t off_wt, off_cs, off_bp, off_g, off_s, off_du, total;
 };
 
 LnPlan make_plan(const mf_lnlinear_args* a, bool backward) {
@@ -33,7 +33,6 @@ LnPlan make_plan(const mf_lnlinear_args* a, bool backward) {
   if (backward) {
     pl.R = ln_row_ranges(a->M, a->K, a->N);
     pl.rows_per_range = (a->M + pl.R - 1) / pl.R;
-    pl.off_wg = off; off += align256((uint64_t)a->K * a->N * es);
     pl.off_g = off; off += align256((uint64_t)pl.R * a->K * a->N * 4);
     pl.off_s = off; off += align256((uint64_t)pl.R * a->N * 4);
     if (swiglu) { pl.off_du = off; off += align256(ln_swiglu_bwd_scratch_elems(a->dtype, a->M, a->K, a->N) * es); }
@@ -101,7 +100,6 @@ LnParams fill(const mf_lnlinear_args* a, const LnPlan& pl, bool backward) {
     p.bprime = reinterpret_cast<float*>(ws + pl.off_bp);
   }
   if (backward) {
-    p.Wg = ws + pl.off_wg;
     p.Gpart = reinterpret_cast<float*>(ws + pl.off_g);
     p.spart = reinterpret_cast<float*>(ws + pl.off_s);
     p.R = pl.R; p.rows_per_range = pl.rows_per_range;
@@ -145,15 +143,17 @@ extern "C" int mf_lnlinear_bwd(const mf_lnlinear_args* a) {
   const LnParams p = fill(a, pl, true);
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   hipError_t e = hipSuccess;
-  // the register-resident dx kernel forms its slice of gamma (.) W itself; every other path reads the prepared copies
-  if (!(a->act == MF_ACT_NONE && ln_bwd_takes_dx_add(a->dtype, a->K, a->N))) {
+  // The dx kernels multiply dOut by the weights as stored and apply gamma to the fp32 products, as the reference does
+  // (fused_layernorm_linear.py:281-306): only the SwiGLU form, which recomputes the pre-activation with the
+  // forward's prepared operands, needs the preparation kernel.
+  if (a->act == MF_ACT_SWIGLU) {
     e = launch_ln_prep(p, false, stream);
     if (e != hipSuccess) return (int)e;
   }
   const void* dY = a->dout;
   if (a->act == MF_ACT_SWIGLU) {
     // recompute the pre-activation tile by tile and turn dh into dU = [da, dg]; where the shape allows it one pass
-    // forms the weight-gradient partials and dU W'^T per column block, and dU never reaches memory
+    // forms the weight-gradient partials and dU W^T per column block, and dU never reaches memory
     e = launch_ln_swiglu_bwd_fused(p, stream);
     if (e != hipErrorNotSupported) return (int)e;
     e = launch_ln_fwd(p, LN_ACT_SWIGLU_BWD, stream);

@@ -29,7 +29,6 @@ struct LnParams {
   float* rstd;         // [M]
   // prepared weights (workspace)
   void* Wt;            // [N, KP]  gamma[k] * W[k, n], transposed, element type of x   (forward)
-  void* Wg;            // [K, N]   gamma[k] * W[k, n], element type of x               (backward dx)
   float* colsum;       // [N] sum_k Wt[n, k]
   float* bprime;       // [N] sum_k beta[k] W[k, n] + b[n]
   // backward
@@ -37,7 +36,7 @@ struct LnParams {
   void* dx;            // [M, K]
   const void* dx_add;  // [M, K] or null: added to dx (residual dx kernel only, see ln_bwd_takes_dx_add)
   void* du;            // SwiGLU backward scratch, ln_swiglu_bwd_scratch_elems elements: [N / 256, M, KP] shares of
-                       // dU W'^T (fused pass) or [M, N] gradient of the pre-activation
+                       // dU W^T (fused pass) or [M, N] gradient of the pre-activation
   void* dW;            // [K, N]   parameter gradients: float, or the element type of x when grads_as_x
   void* db;            // [N] or null
   void* dgamma;        // [K]

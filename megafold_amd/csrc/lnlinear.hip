@@ -84,7 +84,6 @@ __global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
   const T* gamma = reinterpret_cast<const T*>(p.gamma);
   const T* beta = reinterpret_cast<const T*>(p.beta);
   T* Wt = reinterpret_cast<T*>(p.Wt);
-  T* Wg = reinterpret_cast<T*>(p.Wg);
   float cs[8], bp[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) { cs[e] = 0.0f; bp[e] = 0.0f; }
@@ -103,7 +102,6 @@ __global__ void __launch_bounds__(256) ln_prep_kernel(const LnParams p) {
         cs[e] += gwf[e];
         bp[e] += bk * to_f(w[e]);
       }
-      if (Wg) st8<T>(Wg + (int64_t)k * p.N + n0, gw);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) tile[8 * c8 + e][k] = gwf[e];

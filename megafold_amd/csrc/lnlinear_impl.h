@@ -15,9 +15,11 @@
 // column tiles and writes only h = silu(gate) * value.
 //
 // Backward (fused_layernorm_linear.py:226-348, closed forms at 281-306, 345), two kernels, no atomics:
-//   dx:  w = dOut W'^T (contraction over N on the MFMA, W' chunks through LDS, dOut straight from
-//        global), then c1 = mean(x_hat w), c2 = mean(w), dx = (w - x_hat c1 - c2) r in registers: a
-//        lane owns one row, so the two means are register sums plus one lane exchange.
+//   dx:  w = gamma (.) (dOut W^T) (contraction over N on the MFMA with the weights as stored, W chunks through
+//        LDS, dOut straight from global; gamma multiplies the fp32 products, as in the reference, so the
+//        rounding of W' never enters the gradient), then c1 = mean(x_hat w), c2 = mean(w),
+//        dx = (w - x_hat c1 - c2) r in registers: a lane owns one row, so the two means are register sums
+//        plus one lane exchange.
 //   dW:  G = x_hat^T dOut and s = colsum(dOut) per row range (contraction over the rows: both
 //        operands are staged row-major and reach the MFMA through transposing LDS reads), then a small
 //        kernel sums the ranges in a fixed order and forms
@@ -387,6 +389,7 @@ static hipError_t launch_fwd_w(const LnParams& p, hipStream_t stream) {
                                                                                         : (size_t)128 * L::XSTR;
   const size_t smem = (size_t)2 * RB * L::XSTR * sizeof(T) + (size_t)4 * RB * 4 + (size_t)2 * 4 * NTW * 32 * 4 +
                       tail_elems * sizeof(T);
+  if (smem > 160 * 1024) return hipErrorInvalidValue;   // not reached: launch_fwd_k picks forms that fit
   auto kern = ln_fwd_kernel<T, KP, NTW, ACT, WN>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -402,7 +405,10 @@ template <typename T, int KP, int ACT> static hipError_t launch_fwd_k(const LnPa
   const int NOUT = (ACT == LN_ACT_NONE) ? p.N : p.N / 2;
   constexpr bool wide = sizeof(T) == 4 || KP > 128;   // fragments twice as large: halve the resident slice
   if constexpr (ACT == LN_ACT_NONE) {
-    if (NOUT <= 32) return launch_fwd_w<T, KP, 1, ACT, 1>(p, stream);
+    // one column tile, four row blocks per work-group: two staged blocks of 128 rows of 512 bytes would not
+    // fit the LDS next to the weight staging area, such rows take the two-by-two form
+    if constexpr (KP * sizeof(T) <= 256)
+      if (NOUT <= 32) return launch_fwd_w<T, KP, 1, ACT, 1>(p, stream);
     if (NOUT <= 128) return launch_fwd_w<T, KP, 2, ACT, 2>(p, stream);
     if constexpr (wide) {
       return launch_fwd_w<T, KP, 2, ACT, 4>(p, stream);
@@ -453,13 +459,13 @@ template <typename T> hipError_t ln_fwd_dispatch(const LnParams& p, int act, hip
 // =================================================================================================
 // backward: dx
 // =================================================================================================
-// RTW row tiles (of 32 rows) per wavefront share every W' fragment read from LDS, and the work-group
-// streams the whole of W' once per 128 * RTW rows: that stream (from L2, through L1) is as large as
+// RTW row tiles (of 32 rows) per wavefront share every W fragment read from LDS, and the work-group
+// streams the whole of W once per 128 * RTW rows: that stream (from L2, through L1) is as large as
 // dOut itself at RTW = 1, so two tiles per wavefront are used where the registers allow it.
 template <typename T, int KP, int RTW>
 __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_kernel(const LnParams p, const T* __restrict__ dY) {
   using frag = frag_t<T>;
-  constexpr int KPT = KP < 32 ? 32 : KP;       // rows of the W' operand, padded to whole tiles
+  constexpr int KPT = KP < 32 ? 32 : KP;       // rows of the W operand, padded to whole tiles
   constexpr int KT = KPT / 32;
   constexpr int NC = 64;                       // columns of N per staged chunk
   constexpr int UNIT = 16 / (int)sizeof(T);
@@ -472,13 +478,14 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_k
   T* Ws = reinterpret_cast<T*>(smem_raw);      // [2][KPT][WSTR]
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
-  const T* Wg = reinterpret_cast<const T*>(p.Wg);
+  const T* Wsrc = reinterpret_cast<const T*>(p.W);   // the weights as stored; gamma multiplies the fp32 products below
+  const T* gam = reinterpret_cast<const T*>(p.gamma);
   const T* X = reinterpret_cast<const T*>(p.x);
   T* dX = reinterpret_cast<T*>(p.dx);
   const int N = p.N, K = p.K;
   const int nchunks = (N + NC - 1) / NC;
 
-  // W' chunk staging: loads are only issued here (clamped addresses), padding is applied at the stash
+  // W chunk staging: loads are only issued here (clamped addresses), padding is applied at the stash
   frag wr_[PF];
   auto fetch_w = [&](int c) {
 #pragma unroll
@@ -486,7 +493,7 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_k
       const int item = tid + 256 * i;
       const int k = (item < WITEMS ? item : 0) / (NC / 8), nc = item % (NC / 8);
       const int n = c * NC + 8 * nc;
-      wr_[i] = ld8<T>(Wg + (int64_t)(k < K ? k : 0) * N + (n < N ? n : 0));
+      wr_[i] = ld8<T>(Wsrc + (int64_t)(k < K ? k : 0) * N + (n < N ? n : 0));
     }
   };
   auto stash_w = [&](int c, int buf) {
@@ -525,7 +532,7 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_k
           yb[j][s] = ld8<T>(dyrow[j] + (n < N ? n : 0));
         }
     };
-    __syncthreads();          // the previous row block is done with both W' buffers
+    __syncthreads();          // the previous row block is done with both W buffers
     fetch_w(0);
     fetch_y(0);
     stash_w(0, 0);
@@ -570,10 +577,12 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_k
         for (int u = 0; u < 2; ++u) {
           const int k0 = (KPT / 2) * g + 16 * kt + 8 * u;
           const frag xv = k0 < K ? ld8<T>(X + mc[j] * K + k0) : frag_zero<T>();
+          const frag gv = k0 < K ? ld8<T>(gam + k0) : frag_zero<T>();
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float v = k0 < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
             xh[kt][8 * u + e] = v;
+            acc[j][kt][8 * u + e] *= to_f(gv[e]);            // dOut W^T times gamma, in fp32
             s1 += v * acc[j][kt][8 * u + e];
             s2 += acc[j][kt][8 * u + e];
           }
@@ -602,7 +611,7 @@ __global__ void __launch_bounds__(256, KP * sizeof(T) > 256 ? 1 : 2) ln_bwd_dx_k
 
 // -------------------------------------------------------------------------------------------------
 // dx for K <= 128 (four k tiles of 32), N <= 16 * NSTEPS * NH <= 1024 and 16-bit element types.  A
-// wavefront owns one k tile and one of NH halves of N and keeps that slice of W' in registers for the
+// wavefront owns one k tile and one of NH halves of N and keeps that slice of W in registers for the
 // whole kernel (A operand), so the only streams are dOut and x in and dx out.  dOut and x rows are
 // fetched coalesced one block ahead, staged in LDS and read by all wavefronts; with NH = 2 the two
 // halves of a k tile are added through LDS; the LayerNorm backward needs row sums over all K, which the
@@ -622,12 +631,13 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
   static_assert(32 * YCH % NTHR == 0, "whole number of chunks per thread");
 
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T* Ys = reinterpret_cast<T*>(smem_raw);      // [32][YSTR]  dOut block (also used to hand out W')
+  T* Ys = reinterpret_cast<T*>(smem_raw);      // [32][YSTR]  dOut block (also used to hand out W)
   T* Xs = Ys + 32 * YSTR;                      // [32][XSTR]  x block
   T* Os = Xs + 32 * XSTR;                      // [32][XSTR]  dx block
   T* Rs = Os + 32 * XSTR;                      // [32][XSTR]  rows of dx_add (the gradient that skips the operator; ADD only)
   float* part = reinterpret_cast<float*>(Os + (ADD ? 2 : 1) * 32 * XSTR);   // [4][32][2] per-k-tile row sums
   float* pair = part + 4 * 32 * 2;                          // [4][16][64] second half's accumulators (NH = 2)
+  T* gl = reinterpret_cast<T*>(pair + (NH == 2 ? 4 * 16 * 64 : 0));   // [128] gamma, zero past K
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const int kt = w & 3, nh = w >> 2;
@@ -638,7 +648,9 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
   T* dX = reinterpret_cast<T*>(p.dx);
   const T* DR = ADD ? reinterpret_cast<const T*>(p.dx_add) : nullptr;
 
-  // ---- resident slice of W' (rows 32 kt .. 32 kt + 31, columns of half nh), handed out through the
+  if (tid < 16) st8<T>(gl + 8 * tid, 8 * tid < K ? ld8<T>(gam + 8 * tid) : frag_zero<T>());   // published by the barriers below
+
+  // ---- resident slice of W (rows 32 kt .. 32 kt + 31, columns of half nh), handed out through the
   // dOut staging area one k tile at a time
   frag af[NSTEPS];
   for (int ww = 0; ww < 4; ++ww) {
@@ -649,12 +661,8 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
       const int r = item / YCH, c = item % YCH;
       const int k = 32 * ww + r;
       const bool ok = k < K && 8 * c < N;
-      // W' = gamma (.) W formed here, once per work-group, with the rounding of the preparation kernel: the
-      // backward of the plain linear form then needs no preparation launch at all
-      const frag wv = ld8<T>(Wraw + (int64_t)(ok ? k : 0) * N + (ok ? 8 * c : 0));
-      const float gk = to_f(gam[ok ? k : 0]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) tmp[i][e] = (T)(gk * to_f(wv[e]));
+      // the weights as stored: gamma multiplies the fp32 products (below), as the reference applies it
+      tmp[i] = ld8<T>(Wraw + (int64_t)(ok ? k : 0) * N + (ok ? 8 * c : 0));
     }
 #pragma unroll
     for (int i = 0; i < YPF; ++i) {
@@ -761,20 +769,25 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
     }
 
     // LayerNorm backward: a lane of half 0 holds w[m][32 kt + 16 g + 0..15]
-    float xh[16];
     float s1 = 0.0f, s2 = 0.0f;
     if (nh == 0) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int k0 = 32 * kt + 16 * g + 8 * u;
-        const frag xv = ld8<T>(Xs + x * XSTR + k0);
+      for (int q = 0; q < 4; ++q) {
+        // dOut W^T times gamma in fp32, formed where it is used (here and below) instead of once in place (rewriting
+        // the accumulator block costs the compiler a second copy of it); four columns at a time, so that the
+        // operands of one quarter are all that is in registers beside the accumulators
+        using half = typename Frag<T>::half;
+        const int k0 = 32 * kt + 16 * g + 4 * q;
+        const half xq = *reinterpret_cast<const half*>(Xs + x * XSTR + k0);
+        const half gq = *reinterpret_cast<const half*>(gl + k0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float v = k0 + e < K ? (to_f(xv[e]) - mu) * rs : 0.0f;
-          xh[8 * u + e] = v;
-          s1 += v * acc[8 * u + e];
-          s2 += acc[8 * u + e];
+        for (int e = 0; e < 4; ++e) {
+          const float v = k0 + e < K ? (to_f(xq[e]) - mu) * rs : 0.0f;
+          const float wg = acc[4 * q + e] * to_f(gq[e]);
+          s1 += v * wg;
+          s2 += wg;
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
       s1 += __shfl_xor(s1, 32);
       s2 += __shfl_xor(s2, 32);
@@ -787,17 +800,30 @@ __global__ void __launch_bounds__(256 * NH, 2 / NH) ln_bwd_dx_res_kernel(const L
 #pragma unroll
       for (int ww = 0; ww < 4; ++ww) { t1 += part[(ww * 32 + x) * 2]; t2 += part[(ww * 32 + x) * 2 + 1]; }
       const float c1 = t1 / (float)K, c2 = t2 / (float)K;
-      float o[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[i] = (acc[i] - (xh[i] * c1 + c2)) * rs;
-      if constexpr (ADD) {                       // summed in fp32, rounded once below
-        const frag r0 = ld8<T>(Rs + x * XSTR + 32 * kt + 16 * g), r1 = ld8<T>(Rs + x * XSTR + 32 * kt + 16 * g + 8);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { o[i] += to_f(r0[i]); o[8 + i] += to_f(r1[i]); }
-      }
       T* orow = Os + x * XSTR + 32 * kt + 16 * g;
-      st8<T>(orow, cvt8<T>(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]));
-      st8<T>(orow + 8, cvt8<T>(o[8], o[9], o[10], o[11], o[12], o[13], o[14], o[15]));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {                // four columns at a time, as above; x_hat is formed again from the
+        using half = typename Frag<T>::half;       // staged row rather than kept in sixteen registers across the barrier
+        const int k0 = 32 * kt + 16 * g + 4 * q;
+        const half xq = *reinterpret_cast<const half*>(Xs + x * XSTR + k0);
+        const half gq = *reinterpret_cast<const half*>(gl + k0);
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = k0 + e < K ? (to_f(xq[e]) - mu) * rs : 0.0f;
+          o[e] = (acc[4 * q + e] * to_f(gq[e]) - (v * c1 + c2)) * rs;
+        }
+        if constexpr (ADD) {                       // summed in fp32, rounded once below
+          const half rq = *reinterpret_cast<const half*>(Rs + x * XSTR + 32 * kt + 16 * g + 4 * q);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] += to_f(rq[e]);
+        }
+        half oq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) oq[e] = (T)o[e];
+        *reinterpret_cast<half*>(orow + 4 * q) = oq;
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   barrier_keep_vm<63>();
@@ -808,7 +834,7 @@ template <typename T, int NSTEPS, int NH, bool ADD>
 static hipError_t launch_dx_res_a(const LnParams& p, const void* dY, hipStream_t stream) {
   constexpr int NP = 16 * NSTEPS * NH;
   const size_t smem = (size_t)(32 * (NP + 8) + (ADD ? 3 : 2) * 32 * (128 + 8)) * sizeof(T) + 4 * 32 * 2 * 4 +
-                      (NH == 2 ? (size_t)4 * 16 * 64 * 4 : 0);
+                      (NH == 2 ? (size_t)4 * 16 * 64 * 4 : 0) + 128 * sizeof(T);
   const int64_t nrb = (p.M + 31) / 32;
   int64_t gx = (2LL / NH) * num_cu();
   if (gx > nrb) gx = nrb;
@@ -844,12 +870,12 @@ static hipError_t launch_dx_r(const LnParams& p, const void* dY, hipStream_t str
   return hipGetLastError();
 }
 
-// Two row tiles per wavefront halve the W' stream but double the block: the grid runs in whole rounds
+// Two row tiles per wavefront halve the W stream but double the block: the grid runs in whole rounds
 // of 2 * CUs resident work-groups, so the larger block only pays when it does not add a partly
 // filled round (a double block is priced at 1.7 single ones).
 template <typename T, int KP> static hipError_t launch_dx_t(const LnParams& p, const void* dY, hipStream_t stream) {
   if constexpr (sizeof(T) == 2 && KP == 128) {
-    // register-resident W': K in (64, 128], 64 <= N <= 1024
+    // register-resident W: K in (64, 128], 64 <= N <= 1024
     if (p.N >= 64) {
       if (p.N <= 128) return launch_dx_res<T, 8, 1>(p, dY, stream);
       if (p.N <= 256) return launch_dx_res<T, 16, 1>(p, dY, stream);
@@ -1182,7 +1208,7 @@ template <typename T> hipError_t ln_dw_dispatch(const LnParams& p, const void* d
 namespace mf {
 
 // SwiGLU backward in three kernels: the fused pass (weight-gradient partials, and each column block's share of
-// dy = dU W'^T in place of dU itself), the reduction of the partials, and dx from the shares.  Returns
+// dU W^T in place of dU itself), the reduction of the partials, and dx from the shares (times gamma).  Returns
 // hipErrorNotSupported for shapes the fused kernel does not take (the caller then runs the separate kernels).
 // With MF_LN_DU_FORM the fused pass writes dU and the general dx kernel reads it back (kept for comparison).
 template <typename T> hipError_t ln_swiglu_bwd_fused_dispatch(const LnParams& p, hipStream_t stream) {

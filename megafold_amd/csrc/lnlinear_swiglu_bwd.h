@@ -2,8 +2,8 @@
 // gradient of h into dU = [da, dg] (fused_transition.py:44-47) and, in the same pass, use dU for everything that
 // needs it, so that dU itself (M x N elements, eight times the size of x) never reaches HBM:
 //   * the weight-gradient partials G = x_hat^T dU and s = colsum(dU);
-//   * each column block's share of dy = dU W'^T, [rows, K] in the element type of x (PARTS form).  The dx kernel
-//     below adds the N / 256 shares and applies the LayerNorm backward.
+//   * each column block's share of dU W^T, [rows, K] in the element type of x (PARTS form; W as stored).  The dx
+//     kernel below adds the N / 256 shares, multiplies by gamma in fp32 and applies the LayerNorm backward.
 // (With PARTS = false the kernel writes dU instead and the general dx kernel reads it back.)
 //
 // A work-group has eight wavefronts on a block of 32 rows and 128 value + 128 gate columns:
@@ -13,7 +13,7 @@
 //  * wavefronts 4-7 ("consumers") take the tiles one iteration later.  Through transposing LDS reads consumer
 //    w - 4 uses the two tiles of producer w - 4 as the B operand of G[k, n] += x_hat^T[k, m] dU[m, n]
 //    (x_hat: the normalised rows, staged beside the raw ones) and adds those tiles' column sums; with plain row
-//    reads of all four producers' tiles it forms dy^T[k, m] = sum_n W'[k, n] dU[m, n] for k tile w - 4, the W'
+//    reads of all four producers' tiles it forms dy^T[k, m] = sum_n W[k, n] dU[m, n] for k tile w - 4, the W
 //    fragments coming from registers or from a private LDS slot per lane.
 // One producer and one consumer share a SIMD, so that the matrix-pipe and LDS work of the second runs in issue
 // slots the first (bound by the vector ALU: the activation) leaves empty.
@@ -32,7 +32,7 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
   constexpr int RB = 32;
   // normalised rows are read with transposing reads (four consecutive rows per 16 lanes): rows 8 banks apart
   constexpr int XHSTR = (L::XSTR * (int)sizeof(T) / 4) % 64 == 4 ? L::XSTR + 8 : L::XSTR;
-  constexpr int WLDS = KP > 64 ? 15 : 8;            // PARTS: W' fragments per consumer kept in LDS
+  constexpr int WLDS = KP > 64 ? 15 : 8;            // PARTS: W fragments per consumer kept in LDS
   constexpr int OSTR = 32 + 8;                      // row stride of a 32-column tile (elements)
   constexpr int TILE = 32 * OSTR;                   // one da or dg tile
   constexpr int PSET = 4 * TILE + 32;               // tiles of one producer: [2 buffers][da, dg], then 64 bytes that
@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
   float* bpL = csL + 4 * 2 * 32;
   T* Ot = reinterpret_cast<T*>(bpL + 4 * 2 * 32);                  // [4 producers][2 buffers][da, dg][32][OSTR]
   T* Dh = Ot + 4 * PSET;                                           // [4 producers][32][OSTR] incoming gradient
-  T* Wl = Dh + 4 * TILE;                                           // PARTS: [4 consumers][WLDS][64 lanes][8] W' fragments
+  T* Wl = Dh + 4 * TILE;                                           // PARTS: [4 consumers][WLDS][64 lanes][8] W fragments
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, x = l & 31, g = l >> 5;
   const bool producer = w < 4;
@@ -226,8 +226,8 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
     float csum[2] = {0.0f, 0.0f};
 #pragma unroll
     for (int a = 0; a < KT; ++a) { G[a][0] = acc_zero(); G[a][1] = acc_zero(); }
-    // PARTS: rows k = 32 pw .. + 31 of W' for the work-group's 256 columns, resident as A operands of
-    // dy^T[k, m] = sum_n W'[k, n] dU[m, n].  Lane row x supplies k = 32 pw + 16 ((x >> 2) & 1) + 4 (x >> 3) + (x & 3),
+    // PARTS: rows k = 32 pw .. + 31 of W (as stored) for the work-group's 256 columns, resident as A operands of
+    // dy^T[k, m] = sum_n W[k, n] dU[m, n].  Lane row x supplies k = 32 pw + 16 ((x >> 2) & 1) + 4 (x >> 3) + (x & 3),
     // so that the accumulator of lane (m, g) holds the 16 contiguous k = 32 pw + 16 g .. + 15.
     // The first WREG fragments stay in registers; the others are parked in LDS, one 16-byte slot per lane (the
     // registers do not hold all sixteen beside the weight-gradient accumulators).
@@ -235,19 +235,19 @@ __global__ void __launch_bounds__(512, 1) ln_swiglu_bwd_fused_kernel(const LnPar
     frag wgf[PARTS && WREG > 0 ? WREG : 1];
     T* wl = Wl + (pw * WLDS * 64 + l) * 8;
     if constexpr (PARTS) {
-      const T* Wgp = reinterpret_cast<const T*>(p.Wg);
+      const T* Wsrc = reinterpret_cast<const T*>(p.W);       // the weights as stored: gamma is applied to the summed shares
       const int k = 32 * pw + 16 * ((x >> 2) & 1) + 4 * (x >> 3) + (x & 3);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int pp = i >> 2, b = (i >> 1) & 1, st = i & 1;
         const int n = b * Nhalf + (blockIdx.y * 4 + pp) * 32 + 16 * st + 8 * g;
-        const frag wv = k < p.K ? ld8<T>(Wgp + (int64_t)k * p.N + n) : frag_zero<T>();
+        const frag wv = k < p.K ? ld8<T>(Wsrc + (int64_t)k * p.N + n) : frag_zero<T>();
         if (i < WREG) wgf[i] = wv; else st8<T>(wl + (i - WREG) * 64 * 8, wv);
       }
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) once, so that no wait for these loads is placed inside the loop
     }
     // One row block: the weight-gradient products of producer pw's two tiles and, with PARTS, the column block's
-    // share of dy = dU W'^T for k tile pw (all four producers' tiles), in the element type of x, to
+    // share of dU W^T for k tile pw (all four producers' tiles), in the element type of x, to
     // part[blockIdx.y][m][KP] (32 contiguous bytes per lane); the dx kernel adds the column blocks' shares.
     // The dy products form one dependent chain and are issued between the independent weight-gradient products.
     auto consume = [&](int64_t rbx, int fb, const T* xh) {
@@ -368,12 +368,13 @@ __global__ void __launch_bounds__(256) ln_bwd_dx_parts_kernel(const LnParams p, 
     for (int e = 0; e < 8; ++e) wv[e] += to_f(pv[e]);
   }
   const frag xv = live ? ld8<T>(reinterpret_cast<const T*>(p.x) + m * p.K + 8 * dc) : frag_zero<T>();
+  const frag gv = live ? ld8<T>(reinterpret_cast<const T*>(p.gamma) + 8 * dc) : frag_zero<T>();
   const float mu = p.mean[m], rs = p.rstd[m];
   float xh[8], s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     xh[e] = live ? (to_f(xv[e]) - mu) * rs : 0.0f;
-    wv[e] = live ? wv[e] : 0.0f;
+    wv[e] = live ? wv[e] * to_f(gv[e]) : 0.0f;              // the shares are dU W^T: gamma in fp32, as the reference applies it
     s1 += xh[e] * wv[e];
     s2 += wv[e];
   }

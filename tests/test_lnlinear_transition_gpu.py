@@ -54,6 +54,11 @@ SWEEP = [
     ((70000,), 256, 512, torch.bfloat16, True),   # 512-byte rows: one work-group per compute unit, several iterations each
     ((9000,), 128, 256, torch.float32, False),    # the same for fp32 rows
     ((3000,), 256, 64, torch.float32, True),
+    ((53,), 128, 8, torch.float32, True),         # 512-byte rows with a single column tile
+    ((30928,), 32, 1024, torch.bfloat16, True),   # wide N on a short row: dx takes gamma in fp32 (a dx through the
+    ((12736,), 56, 520, torch.bfloat16, True),    # rounded gamma (.) W misses the element-wise bar on these three)
+    ((2639,), 64, 1024, torch.bfloat16, False),
+    ((700,), 256, 24, torch.bfloat16, False),
     ((100,), 768, 768, torch.float32, True),      # K beyond the kernels: same eager expression as the reference's fallback
 ]
 
