@@ -376,3 +376,38 @@ def test_config5_peak_activation_memory():
     again = run_op({k_: v_.detach() for k_, v_ in dev.items()})
     assert torch.equal(again[1], q.grad) and torch.equal(again[2], k.grad) and torch.equal(again[3], v.grad)
     assert torch.equal(again[4], dB)
+
+
+@pytest.mark.gpu
+def test_tensors_beyond_two_to_the_31_elements_match_their_row_slices():
+    """[1, 17000, 512, 8, 32] bf16: 2.2e9 elements (4.4 GB) per tensor, so that element and byte offsets of the later
+    rows pass 2^31.  The rows n are independent problems: O, dQ, dK, dV of the full call must equal, bit for bit, those
+    of calls on row slices (whose offsets are small), near the end of the tensors and over both halves; dBias of the
+    halves must add up to the full one within the rounding of the 16-bit outputs."""
+    B, N, S, H, D = 1, 17000, 512, 8, 32
+    torch.manual_seed(0)
+    mk = lambda *sh: torch.randn(*sh, device="cuda").to(torch.bfloat16)
+    q, k, v, dO = (mk(B, N, S, H, D) for _ in range(4))
+    bias = mk(B, 1, H, S, S)
+    mask = torch.zeros(B, N, 1, 1, S, device="cuda")
+    mask[..., S - 37:] = float("-inf")
+
+    def run(sl):
+        qq, kk, vv = (t[:, sl].detach().clone().requires_grad_() for t in (q, k, v))
+        bb = bias.detach().clone().requires_grad_()
+        o = TritonEvoformer(qq, kk, vv, mask[:, sl], bb)
+        o.backward(dO[:, sl])
+        return o.detach(), qq.grad, kk.grad, vv.grad, bb.grad
+
+    full = run(slice(0, N))
+    assert all(bool(torch.isfinite(t.float()).all()) for t in full)
+    halves = []
+    for sl in (slice(N - 8, N), slice(N - 305, N - 295), slice(0, N // 2), slice(N // 2, N)):
+        part = run(sl)
+        for name, a, b in zip(("O", "dQ", "dK", "dV"), full[:4], part[:4]):
+            assert torch.equal(a[:, sl], b), "%s of rows %s differs from the sliced call" % (name, sl)
+        if sl.stop - sl.start == N // 2:
+            halves.append(part[4].float())
+        del part
+    want = halves[0] + halves[1]
+    torch.testing.assert_close(full[4].float(), want, rtol=2 ** -7, atol=2 ** -7 * float(want.abs().max()))

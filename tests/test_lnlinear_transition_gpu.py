@@ -295,3 +295,40 @@ def test_backward_dx_add_matches_the_separate_sum(K, N, act, dtype):
     for a, b in zip(got[1:], want[1:]):                          # parameter gradients do not see it
         if a is not None:
             assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["lnlinear", "transition"])
+def test_outputs_beyond_two_to_the_31_elements_match_their_row_slices(kind):
+    """M = 2 200 001 rows of K = 128 into N = 1024 columns: 2.25e9 elements of output (and of incoming gradient) in the
+    plain form, as many of pre-activation in the transition.  Rows are independent: out and dx of the full call must
+    equal, bit for bit, those of calls on row slices near the end and on both halves; the parameter gradients of the
+    halves must add up to the full ones within the rounding of the 16-bit results."""
+    torch.manual_seed(0)
+    dt, M, K = torch.bfloat16, 2_200_001, 128
+    if kind == "lnlinear":
+        mod, n_out = LayernormLinear(K, 1024, has_linear_bias=True, device="cuda", dtype=dt), 1024
+    else:
+        mod, n_out = FusedTransition(K, 4, device="cuda", dtype=dt), K
+    x = torch.randn(M, K, device="cuda").to(dt)
+    dy = torch.randn(M, n_out, device="cuda").to(dt)
+
+    def run(sl):
+        xx = x[sl].detach().clone().requires_grad_()
+        for p in mod.parameters():
+            p.grad = None
+        y = mod(xx)
+        y.backward(dy[sl])
+        return y.detach(), xx.grad, [p.grad.float().clone() for p in mod.parameters()]
+
+    full = run(slice(0, M))
+    halves = []
+    for sl in (slice(M - 1000, M), slice(M - 70001, M - 69000), slice(0, M // 2), slice(M // 2, M)):
+        part = run(sl)
+        assert torch.equal(full[0][sl], part[0]), "out of rows %s differs from the sliced call" % (sl,)
+        assert torch.equal(full[1][sl], part[1]), "dx of rows %s differs from the sliced call" % (sl,)
+        if sl.stop - sl.start >= M // 2:
+            halves.append(part[2])
+        del part
+    for a, b, c in zip(full[2], halves[0], halves[1]):
+        torch.testing.assert_close(a, b + c, rtol=2 ** -6, atol=2 ** -6 * float(a.abs().max()))
