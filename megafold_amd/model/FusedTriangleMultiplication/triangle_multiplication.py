@@ -17,6 +17,9 @@ What runs, per call (one ``torch.autograd.Function``, nothing channel-last is ev
 4. ``mf_channels_first_to_last`` back to rows, fused LayerNorm -> Linear ``dh -> dim``, and the sigmoid output
    gate read in place from Y's last columns (``mf_sigmoid_gate_fwd``).
 
+Widths other than 64 and 128 run the same expression from the two fused LayerNorm -> Linear
+modules and PyTorch operations on the GPU (``TriangleMultiplication._composed``).
+
 Backward mirrors it with ``mf_sigmoid_gate_bwd``, ``mf_lnlinear_bwd``, ``mf_channels_last_to_first``, two batched
 GEMMs, ``mf_trimul_pack_bwd`` (GLU and mask backward fused into the move back, written straight into the
 columns of dY) and one ``mf_lnlinear_bwd``.
@@ -174,13 +177,31 @@ class TriangleMultiplication(nn.Module):
         self.to_out = nn.Sequential(LayernormLinear(dim_hidden, dim, has_linear_bias=False),
                                     Dropout(dropout, dropout_type=dropout_type))
 
+    def _composed(self, x: torch.Tensor, mask: Optional[torch.Tensor]) -> torch.Tensor:
+        """The block for the widths the layout kernels do not take (they move rows of 64 or 128 hidden channels): the two ``LayernormLinear`` modules as they are, and the gated-linear unit, pair mask,
+        contraction and output gate of megafold.py:475-491 as PyTorch operations on the GPU, with PyTorch's autograd."""
+        dh = self.dim_hidden
+        y = self.combined(x)
+        gate = torch.sigmoid(y[..., 4 * dh:])
+        left, right = torch.nn.functional.glu(y[..., :4 * dh], dim=-1).chunk(2, dim=-1)
+        if mask is not None:
+            keep = (mask[:, :, None] & mask[:, None, :]).unsqueeze(-1).to(left.dtype)
+            left, right = left * keep, right * keep
+        eq = "bikd,bjkd->bijd" if self.mix == "outgoing" else "bkjd,bkid->bijd"
+        out = torch.einsum(eq, left, right).contiguous()
+        return self.to_out[0](out) * gate
+
     def forward(self, x: torch.Tensor, mask: Optional[torch.Tensor] = None, add_residual: bool = False) -> torch.Tensor:
         dim, dh = x.shape[-1], self.dim_hidden
         dtype = torch.bfloat16 if torch.is_autocast_enabled() else x.dtype
         if not x.is_cuda:
             raise RuntimeError("TriangleMultiplication runs on the GPU only (got device %s)" % x.device)
-        if dh != dim or dh not in (64, 128) or not fused_shape_supported(dim, 5 * dh, dtype):
-            raise ValueError("unsupported shape for the fused block: dim=%d dim_hidden=%d" % (dim, dh))
+        if dh != dim:        # the reference multiplies the [.., dim] projection by a [.., dim_hidden] gate (megafold.py:491)
+            raise ValueError("dim_hidden (%d) must equal dim (%d): the output gate has dim_hidden columns" % (dh, dim))
+        if dh not in (64, 128) or not fused_shape_supported(dim, 5 * dh, dtype):
+            out = self._composed(x, mask)         # other widths: the same expression from the module's own parts
+            out = self.to_out[1](out)
+            return out + x if add_residual else out
         c, o = self.combined, self.to_out[0]
         drop = self.to_out[1]
         # the fused sum adds in the compute dtype: under autocast an fp32 residual stream stays fp32 (x + block(x)

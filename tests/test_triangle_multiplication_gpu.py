@@ -94,6 +94,8 @@ CASES = [
     (1, 29, 64, 4, "outgoing", torch.float16),
     (1, 40, 128, 3, "incoming", torch.float32),
     (1, 21, 64, 2, "outgoing", torch.float32),
+    (1, 26, 32, 3, "outgoing", torch.bfloat16),        # widths the layout kernels do not take: the composed path
+    (2, 19, 96, 0, "incoming", torch.float32),
 ]
 
 
@@ -197,3 +199,4 @@ def test_block_against_golden_fixture(mix):
         # out, dx element-wise at the fp32 bar; the weight gradients are sums over 144 rows
         atol = 1e-5 if name in ("out", "dx") else 1e-5 * 12
         torch.testing.assert_close(t.detach().cpu(), want, rtol=1e-4, atol=atol, msg=lambda m_, n=name: "%s: %s" % (n, m_))
+
